@@ -28,7 +28,7 @@
 //     under the tail of the QKV stream, which is the k / v rows; the token of the step itself is folded in by the merging wave
 //     (q . k_new, one more term of the online softmax), so that only "k / v granules -> merge -> publish -> sweep" follows the
 //     end of the QKV stream (Qwen3-8B: 2690 -> 2625 us per launch; polling q a batch earlier, or publishing through the
-//     scalar cache -- s_store glc + s_dcache_wb, 0.4 us per idle hop in tools/probes/hop_probe.hip -- both measured slower).
+//     scalar data cache instead of vector stores, both measured slower).
 //   * The residual stream row r is owned by the same lane of the same wave in o_proj and down_proj and lives in LDS.
 // Every spin is bounded; a timeout raises ctl[1], later launches return at once, and the host reports the code.
 #include <cstdio>
