@@ -136,8 +136,10 @@ class Model:
     def _opts(device=0, max_seq_len=0, max_seqs=0, kv_block_size=0, kv_pool_tokens=0, use_graph=0,
               tp_rank=0, tp_size=1, tp_unique_id: Optional[bytes] = None, prefill_chunk=0, prefill_split=0,
               kv_dtype="f16", isq: Optional[str] = None, engine=0, debug_tp_local=False, debug_force_rccl=False,
-              tp_in_process=False, tp_devices: Optional[List[int]] = None, tp_collective: Optional[str] = None):
+              tp_in_process=False, tp_devices: Optional[List[int]] = None, tp_collective: Optional[str] = None,
+              compute_dtype: str = "bfloat16"):
         o = _lib.CmOpts()
+        o.compute_dtype = {"bfloat16": 0, "bf16": 0, "float32": 1, "f32": 1}[compute_dtype]     # layer-list decoders only
         o.abi_version = _lib.CM_ABI_VERSION
         o.device, o.tp_rank, o.tp_size = device, tp_rank, tp_size
         o.max_seq_len, o.max_seqs, o.kv_block_size = max_seq_len, max_seqs, kv_block_size
@@ -309,6 +311,40 @@ class Model:
             self._h, sa.ctypes.data_as(C.POINTER(C.c_int32)), ptrs, lens, n,
             out.ctypes.data_as(C.POINTER(C.c_float)) if want_logits else None, g.ctypes.data_as(C.POINTER(C.c_uint32))))
         return out, g
+
+    def step_batch(self, items, want_logits=True):
+        """cm_step_batch: one step of a layer-list decoder.  items: (seq, tokens, want) with want = positions inside the portion
+        whose logits are asked for (None: the last one).  All items run as one batch.  Returns ([rows, V] logits or None,
+        greedy ids [rows]) in the order of the items and their wanted positions."""
+        n = len(items)
+        arr = (_lib.CmStepItem * n)()
+        keep, rows = [], 0
+        for i, (seq, toks, want) in enumerate(items):
+            ta = np.ascontiguousarray(np.asarray(toks, dtype=np.uint32))
+            arr[i].seq, arr[i].tokens, arr[i].n_tokens = int(seq), ta.ctypes.data_as(C.POINTER(C.c_uint32)), ta.size
+            if want is None:
+                arr[i].n_want, arr[i].want = -1, None
+                rows += 1
+            else:
+                wa = np.ascontiguousarray(np.asarray(want, dtype=np.int32))
+                arr[i].n_want, arr[i].want = wa.size, wa.ctypes.data_as(C.POINTER(C.c_int32))
+                rows += wa.size
+                keep.append(wa)
+            keep.append(ta)
+        out = np.empty((rows, self.vocab_size), dtype=np.float32) if want_logits else None
+        g = np.empty(max(rows, 1), dtype=np.uint32)
+        self._check(self._lib.cm_step_batch(
+            self._h, arr, n, out.ctypes.data_as(C.POINTER(C.c_float)) if want_logits and rows else None,
+            g.ctypes.data_as(C.POINTER(C.c_uint32))))
+        return out, g[:rows]
+
+    def layer_capture(self, on: bool = True) -> None:
+        """Layer-list decoders: keep the residual stream after every layer of every pass (read it with layer_rows())."""
+        self.debug_set("lay_capture", 1 if on else 0)
+
+    def layer_rows(self) -> np.ndarray:
+        n = int(self.debug_read("lay_layers_len", 1)[0])
+        return self.debug_read("lay_layers", n) if n else np.zeros(0, np.float32)
 
     def step_batch_decode(self, seqs: Sequence[int], tokens: Sequence[int], want_logits=True):
         """step_batch_decode (backend.rs:107-121): returns ([N,1,V] logits or None, greedy ids [N])."""

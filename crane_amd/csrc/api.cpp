@@ -131,7 +131,11 @@ int cm_create(const char* model_dir, const cm_opts* opts, cm_model** out) {
         catch (const std::exception& e) { throw CmError(CM_ERR_IO, e.what()); }
         h = new cm_model();
         create_ranks(h, cfg, opts, [&](Model& m) {
-            if (gguf) cm::load_from_gguf(m, path);
+            if (m.layered) {
+                if (gguf) throw CmError(CM_ERR_UNSUPPORTED, "GGUF files hold no layer-list decoder");
+                cm::load_layered_from_dir(m, path);
+            }
+            else if (gguf) cm::load_from_gguf(m, path);
             else { cm::load_from_dir(m, path); apply_isq(m); }
         });
     });
@@ -146,7 +150,10 @@ int cm_create_synthetic(const char* config_json, uint64_t seed, const cm_opts* o
     cm_model* h = nullptr;
     int rc = guard(nullptr, [&] {
         h = new cm_model();
-        create_ranks(h, config_json, opts, [&](Model& m) { cm::load_synthetic(m, seed); apply_isq(m); });
+        create_ranks(h, config_json, opts, [&](Model& m) {
+            if (m.layered) { cm::load_layered_synthetic(m, seed); return; }
+            cm::load_synthetic(m, seed); apply_isq(m);
+        });
     });
     if (rc != CM_OK) { delete h; return rc; }
     *out = h;
@@ -358,6 +365,17 @@ int cm_decode_batch(cm_model* h, const int32_t* seqs, const uint32_t* last_token
     });
 }
 
+int cm_step_batch(cm_model* h, const cm_step_item* items, size_t n, float* logits_out, uint32_t* greedy_out) {
+    if (!h) return CM_ERR_INVALID;
+    return guard(h, [&] {
+        if (h->grp) throw CmError(CM_ERR_UNSUPPORTED, "cm_step_batch: not available on an in-process tensor-parallel group");
+        if (!items || n == 0) throw CmError(CM_ERR_INVALID, "empty step");
+        std::vector<Model::StepItem> it(n);
+        for (size_t i = 0; i < n; ++i) it[i] = Model::StepItem{items[i].seq, items[i].tokens, items[i].n_tokens, items[i].want, items[i].n_want};
+        h->m.step_batch(it.data(), n, logits_out, greedy_out);
+    });
+}
+
 int64_t cm_image_token_id(const cm_model* h) { return (h && h->m.vcfg.present) ? (int64_t)h->m.vcfg.image_token : -1; }
 
 int cm_vision_encode(cm_model* h, const float* pixel_values, size_t n_patches, const uint32_t* grid_thw, size_t n_images,
@@ -476,6 +494,8 @@ int cm_debug_read(cm_model* h, const char* what, float* out, size_t n) {
         const float* src = nullptr;
         size_t avail = 0;
         const std::string w = w0;
+        if (w == "lay_layers_len") { if (n < 1) throw CmError(CM_ERR_INVALID, "n < 1"); out[0] = (float)mp->layered_capture(nullptr, 0); return; }
+        if (w == "lay_layers") { (void)mp->layered_capture(out, n); return; }
         // (the persistent kernel never runs under tensor parallelism and the tower's debug buffers live on rank 0: no '@r' form)
         if (mp != &h->m && (w == "engine_trace" || w.rfind("eng_", 0) == 0 || w == "vision_ms" || w == "deepstack"))
             throw CmError(CM_ERR_INVALID, "cm_debug_read: '" + w + "' has no per-rank form");
@@ -553,7 +573,8 @@ int cm_debug_set(cm_model* h, const char* key, int64_t value) {
     if (!h || !key) return CM_ERR_INVALID;
     return guard_all(h, [&](Model& mm, bool) {
         const std::string k = key;
-        if (k == "no_prefill") mm.no_prefill = value != 0;
+        if (k == "lay_capture") mm.layered_set_capture(value != 0);
+        else if (k == "no_prefill") mm.no_prefill = value != 0;
         else if (k == "quant_prefill") mm.quant_prefill = value != 0;
         else if (k == "prefill_q8") {       // before the first prompt pass of the handle: 0 = prompts over Q8_0-layout weights on the dequantised-to-bf16 GEMMs
             if (mm.pX != nullptr) throw CmError(CM_ERR_INVALID, "prefill_q8: set before the first prompt pass");

@@ -1,0 +1,657 @@
+// Kernels of the layer-list decoders (layered.h): every mechanism takes its sizes and constants as arguments.
+// What the model's definition asks for in 32 bits is f32 here in both number formats: residual stream, norms, positions,
+// attention scores and softmax, the linear-attention state and its decay powers, router logits.  The bfloat16 format rounds the
+// A operand of the projections (matrix cores, f32 accumulation) and the cached keys; the float32 format rounds nothing.
+#include <hip/hip_runtime.h>
+
+#include "dev_common.h"
+#include "layered.h"
+
+namespace cm {
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+__device__ __forceinline__ float lay_act(float v, int act) {
+    switch (act) {
+        case LACT_SILU: return v / (1.f + __expf(-v));
+        case LACT_SIGMOID: return 1.f / (1.f + __expf(-v));
+        case LACT_GELU_TANH: {
+            const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+            return 0.5f * v * (1.f + tanhf(u));
+        }
+        default: return v;
+    }
+}
+
+// sum over the block (blockDim.x a multiple of 64, every thread calls); red: >= blockDim.x / 64 floats of LDS
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t += red[i];
+    __syncthreads();
+    return t;
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// row norms
+// ------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void lay_rms_rows_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
+                                                           const float* __restrict__ w, float* __restrict__ out, int W, float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    const float* xr = x + (size_t)(rows ? rows[r] : r) * W;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) { const float v = xr[c]; ss += v * v; }
+    ss = block_sum(ss, red);
+    const float rs = 1.f / sqrtf(ss / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += 256) out[(size_t)r * W + c] = xr[c] * rs * w[c];
+}
+void launch_lay_rms_rows(const float* x, const int32_t* rows, const float* w, float* out, int n_rows, int W, float eps, hipStream_t s) {
+    if (n_rows <= 0) return;
+    hipLaunchKernelGGL(lay_rms_rows_kernel, dim3((unsigned)n_rows), dim3(256), 0, s, x, rows, w, out, W, eps);
+}
+
+__global__ __launch_bounds__(256) void lay_rms_gate_kernel(const float* __restrict__ o, const float* __restrict__ gate, int ldg,
+                                                           const float* __restrict__ w, float* __restrict__ out, int N, float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    const float* orow = o + (size_t)r * N;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < N; c += 256) { const float v = orow[c]; ss += v * v; }
+    ss = block_sum(ss, red);
+    const float rs = 1.f / sqrtf(ss / (float)N + eps);
+    for (int c = threadIdx.x; c < N; c += 256) out[(size_t)r * N + c] = orow[c] * rs * w[c] * gate[(size_t)r * ldg + c];
+}
+void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s) {
+    if (T <= 0) return;
+    hipLaunchKernelGGL(lay_rms_gate_kernel, dim3((unsigned)T), dim3(256), 0, s, o, gate, ldg, w, out, N, eps);
+}
+
+__global__ __launch_bounds__(256) void lay_post_norm_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ w,
+                                                            float mult, float eps, int W, const float* __restrict__ wsel, int top) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float v;
+        if (wsel) {
+            v = 0.f;
+            for (int k = 0; k < top; ++k) v += wsel[(size_t)r * top + k] * y[((size_t)r * top + k) * W + c];
+        } else v = y[(size_t)r * W + c];
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float rs = 1.f / sqrtf(ss / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float v;
+        if (wsel) {
+            v = 0.f;
+            for (int k = 0; k < top; ++k) v += wsel[(size_t)r * top + k] * y[((size_t)r * top + k) * W + c];
+        } else v = y[(size_t)r * W + c];
+        x[(size_t)r * W + c] += mult * (v * rs * w[c]);
+    }
+}
+void launch_lay_post_norm(float* x, const float* y, const float* w, float mult, float eps, int T, int W, const float* wsel, int top,
+                          hipStream_t s) {
+    if (T <= 0) return;
+    hipLaunchKernelGGL(lay_post_norm_kernel, dim3((unsigned)T), dim3(256), 0, s, x, y, w, mult, eps, W, wsel, top);
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// short causal convolution in front of a sublayer: out_t = h_t + sum_j cw[:, j] h_(t - taps + 1 + j)
+// tail of a sequence = its last taps - 1 inputs, oldest first: [taps - 1][W]
+// ------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void lay_canon_kernel(const float* __restrict__ h, float* __restrict__ out, const float* __restrict__ cw,
+                                                        const float* __restrict__ conv_pool, size_t slot_stride, size_t off,
+                                                        const LaySegDev* __restrict__ segs, const int32_t* __restrict__ rowseg, int W, int taps) {
+    const int r = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= W) return;
+    const LaySegDev sg = segs[rowseg[r]];
+    const int local = r - sg.row0;
+    const float* tail = conv_pool + (size_t)sg.slot * slot_stride + off;
+    float acc = h[(size_t)r * W + c];
+    for (int j = 0; j < taps; ++j) {
+        const int src = local - (taps - 1) + j;
+        const float v = src >= 0 ? h[(size_t)(sg.row0 + src) * W + c] : tail[(size_t)(taps - 1 + src) * W + c];
+        acc += cw[(size_t)c * taps + j] * v;
+    }
+    out[(size_t)r * W + c] = acc;
+}
+void launch_lay_canon(const float* h, float* out, const float* cw, const float* conv_pool, size_t slot_stride, size_t off,
+                      const LaySegDev* segs, const int32_t* rowseg, int T, int W, int taps, hipStream_t s) {
+    if (T <= 0) return;
+    hipLaunchKernelGGL(lay_canon_kernel, dim3((unsigned)T, (unsigned)((W + 255) / 256)), dim3(256), 0, s, h, out, cw, conv_pool, slot_stride,
+                       off, segs, rowseg, W, taps);
+}
+
+// new tail = last taps - 1 entries of (old tail ++ the portion's inputs).  In place: entry k reads entry n + k > k of the old tail,
+// and a thread touches its own channel only.
+__global__ __launch_bounds__(256) void lay_canon_tail_kernel(const float* __restrict__ h, float* __restrict__ conv_pool, size_t slot_stride,
+                                                             size_t off, const LaySegDev* __restrict__ segs, int W, int taps) {
+    const LaySegDev sg = segs[blockIdx.x];
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= W) return;
+    float* tail = conv_pool + (size_t)sg.slot * slot_stride + off;
+    for (int k = 0; k < taps - 1; ++k) {
+        const int idx = sg.n + k;
+        tail[(size_t)k * W + c] = idx < taps - 1 ? tail[(size_t)idx * W + c] : h[(size_t)(sg.row0 + idx - (taps - 1)) * W + c];
+    }
+}
+void launch_lay_canon_tail(const float* h, float* conv_pool, size_t slot_stride, size_t off, const LaySegDev* segs, int nseg, int W,
+                           int taps, hipStream_t s) {
+    if (nseg <= 0 || taps <= 1) return;
+    hipLaunchKernelGGL(lay_canon_tail_kernel, dim3((unsigned)nseg, (unsigned)((W + 255) / 256)), dim3(256), 0, s, h, conv_pool, slot_stride,
+                       off, segs, W, taps);
+}
+
+// decode rows (one token per sequence): norm, convolution and tail shift of a row by the one block that owns its sequence
+__global__ __launch_bounds__(256) void lay_norm_canon_decode_kernel(const float* __restrict__ x, const float* __restrict__ nw, float eps,
+                                                                    float* __restrict__ out, const float* __restrict__ cw,
+                                                                    float* __restrict__ conv_pool, size_t slot_stride, size_t off,
+                                                                    const LaySegDev* __restrict__ segs, int W, int taps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    const LaySegDev sg = segs[r];
+    const float* xr = x + (size_t)sg.row0 * W;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) { const float v = xr[c]; ss += v * v; }
+    ss = block_sum(ss, red);
+    const float rs = 1.f / sqrtf(ss / (float)W + eps);
+    float* tail = conv_pool + (size_t)sg.slot * slot_stride + off;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float hv = xr[c] * rs * nw[c];
+        float acc = hv + cw[(size_t)c * taps + (taps - 1)] * hv;
+        for (int j = 0; j < taps - 1; ++j) {
+            const float tv = tail[(size_t)j * W + c];
+            acc += cw[(size_t)c * taps + j] * tv;
+            if (j > 0) tail[(size_t)(j - 1) * W + c] = tv;
+        }
+        if (taps > 1) tail[(size_t)(taps - 2) * W + c] = hv;
+        out[(size_t)sg.row0 * W + c] = acc;
+    }
+}
+void launch_lay_norm_canon_decode(const float* x, const float* nw, float eps, float* out, const float* cw, float* conv_pool,
+                                  size_t slot_stride, size_t off, const LaySegDev* segs, int T, int W, int taps, hipStream_t s) {
+    if (T <= 0) return;
+    hipLaunchKernelGGL(lay_norm_canon_decode_kernel, dim3((unsigned)T), dim3(256), 0, s, x, nw, eps, out, cw, conv_pool, slot_stride, off,
+                       segs, W, taps);
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// projections: C[p][n] = epilogue(sum_k A[row(p)][k] W[n][k] + bias[n])
+// 64 x 64 outputs per block of 256 threads; any M, N, K (tiles are zero-filled past the edges)
+// ------------------------------------------------------------------------------------------------------------------
+constexpr int LG_BM = 64, LG_BN = 64;
+
+struct LgTile { int p0, rows, n0; const uint16_t* W; const uint16_t* W2; };
+
+__device__ __forceinline__ bool lg_tile(const LGemmArgs& a, LgTile& t) {
+    const int g = blockIdx.z;
+    int base = 0, rows = a.M;
+    if (a.grp_off) { base = a.grp_off[g]; rows = a.grp_off[g + 1] - base; }
+    const int m0 = blockIdx.x * LG_BM;
+    if (m0 >= rows) return false;
+    t.p0 = base + m0;
+    t.rows = min(LG_BM, rows - m0);
+    t.n0 = blockIdx.y * LG_BN;
+    t.W = a.W + (size_t)g * a.w_stride;
+    t.W2 = a.W2 ? a.W2 + (size_t)g * a.w_stride : nullptr;
+    return true;
+}
+
+__device__ __forceinline__ void lg_store(const LGemmArgs& a, int p, int n, float v, float v2, bool dual) {
+    if (a.bias) v += a.bias[n];
+    if (dual) v = lay_act(v, a.act) * v2;
+    else v = lay_act(v, n < a.act_split ? a.act : a.act2);
+    const size_t row = a.c_idx ? (size_t)a.c_idx[p] : (size_t)p;
+    a.C[row * a.ldc + n] = v;
+}
+
+// f32 FMA form: 4 x 4 outputs per thread, k in steps of 16
+template <bool DUAL>
+__global__ __launch_bounds__(256) void lgemm_f32_kernel(LGemmArgs a) {
+    constexpr int BK = 16;
+    __shared__ float As[BK][LG_BM + 4];
+    __shared__ float Bs[BK][LG_BN + 4];
+    __shared__ float B2s[DUAL ? BK : 1][LG_BN + 4];
+    __shared__ int arow[LG_BM];
+    LgTile t;
+    if (!lg_tile(a, t)) return;
+    const int tid = threadIdx.x;
+    if (tid < LG_BM) {
+        int ar = -1;
+        if (tid < t.rows) { const int p = t.p0 + tid; ar = a.a_idx ? a.a_idx[p] / a.a_div : p; }
+        arow[tid] = ar;
+    }
+    __syncthreads();
+    const int ty = tid >> 4, tx = tid & 15;
+    float acc[4][4] = {}, acc2[4][4] = {};
+    for (int k0 = 0; k0 < a.K; k0 += BK) {
+        for (int i = 0; i < 4; ++i) {
+            const int idx = tid + i * 256, r = idx >> 4, kk = idx & 15, k = k0 + kk;
+            const int ar = arow[r];
+            As[kk][r] = (ar >= 0 && k < a.K) ? a.A[(size_t)ar * a.lda + k] : 0.f;
+            const int n = t.n0 + r;
+            const bool ok = n < a.N && k < a.K;
+            Bs[kk][r] = ok ? bf16_to_f32(t.W[(size_t)n * a.K + k]) : 0.f;
+            if (DUAL) B2s[kk][r] = ok ? bf16_to_f32(t.W2[(size_t)n * a.K + k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK; ++kk) {
+            float av[4], bv[4], b2[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { av[i] = As[kk][ty * 4 + i]; bv[i] = Bs[kk][tx * 4 + i]; if (DUAL) b2[i] = B2s[kk][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+                    if (DUAL) acc2[i][j] = fmaf(av[i], b2[j], acc2[i][j]);
+                }
+        }
+        __syncthreads();
+    }
+    for (int i = 0; i < 4; ++i) {
+        const int r = ty * 4 + i;
+        if (r >= t.rows) continue;
+        for (int j = 0; j < 4; ++j) {
+            const int n = t.n0 + tx * 4 + j;
+            if (n < a.N) lg_store(a, t.p0 + r, n, acc[i][j], acc2[i][j], DUAL);
+        }
+    }
+}
+
+// bfloat16 form: A rounded to bfloat16 on its way into LDS, four waves of one 32 x 32 x 8 matrix-core tile each, k in steps of 32
+template <bool DUAL>
+__global__ __launch_bounds__(256) void lgemm_bf16_kernel(LGemmArgs a) {
+    constexpr int BK = 32, LDS_K = BK + 8;
+    __shared__ __attribute__((aligned(16))) uint16_t As[LG_BM][LDS_K];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[LG_BN][LDS_K];
+    __shared__ __attribute__((aligned(16))) uint16_t B2s[DUAL ? LG_BN : 1][LDS_K];
+    __shared__ int arow[LG_BM];
+    LgTile t;
+    if (!lg_tile(a, t)) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid < LG_BM) {
+        int ar = -1;
+        if (tid < t.rows) { const int p = t.p0 + tid; ar = a.a_idx ? a.a_idx[p] / a.a_div : p; }
+        arow[tid] = ar;
+    }
+    __syncthreads();
+    const int wm = wave >> 1, wn = wave & 1;
+    f32x16 acc = {}, acc2 = {};
+    const int lr = tid >> 2, ks = (tid & 3) * 8;         // this thread stages 8 consecutive k of row lr
+    const bool vecA = (a.lda % 4) == 0 && ((uintptr_t)a.A % 16) == 0;
+    const bool vecW = (a.K % 8) == 0 && ((uintptr_t)t.W % 16) == 0 && (!DUAL || ((uintptr_t)t.W2 % 16) == 0);
+    for (int k0 = 0; k0 < a.K; k0 += BK) {
+        const int k = k0 + ks;
+        {
+            float v[8];
+            const int ar = arow[lr];
+            if (ar >= 0 && vecA && k + 8 <= a.K) {
+                const float4 x0 = *(const float4*)(a.A + (size_t)ar * a.lda + k);
+                const float4 x1 = *(const float4*)(a.A + (size_t)ar * a.lda + k + 4);
+                v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
+            } else {
+                for (int i = 0; i < 8; ++i) v[i] = (ar >= 0 && k + i < a.K) ? a.A[(size_t)ar * a.lda + k + i] : 0.f;
+            }
+            u32x4 pk;
+            pk.x = pack_bf16x2(v[0], v[1]); pk.y = pack_bf16x2(v[2], v[3]); pk.z = pack_bf16x2(v[4], v[5]); pk.w = pack_bf16x2(v[6], v[7]);
+            *(u32x4*)&As[lr][ks] = pk;
+        }
+        {
+            const int n = t.n0 + lr;
+            u32x4 pk = {0u, 0u, 0u, 0u}, pk2 = {0u, 0u, 0u, 0u};
+            if (n < a.N) {
+                if (vecW && k + 8 <= a.K) {
+                    pk = *(const u32x4*)(t.W + (size_t)n * a.K + k);
+                    if (DUAL) pk2 = *(const u32x4*)(t.W2 + (size_t)n * a.K + k);
+                } else {
+                    uint16_t e[8], e2[8];
+                    for (int i = 0; i < 8; ++i) {
+                        e[i] = k + i < a.K ? t.W[(size_t)n * a.K + k + i] : (uint16_t)0;
+                        e2[i] = (DUAL && k + i < a.K) ? t.W2[(size_t)n * a.K + k + i] : (uint16_t)0;
+                    }
+                    pk.x = e[0] | ((uint32_t)e[1] << 16); pk.y = e[2] | ((uint32_t)e[3] << 16);
+                    pk.z = e[4] | ((uint32_t)e[5] << 16); pk.w = e[6] | ((uint32_t)e[7] << 16);
+                    pk2.x = e2[0] | ((uint32_t)e2[1] << 16); pk2.y = e2[2] | ((uint32_t)e2[3] << 16);
+                    pk2.z = e2[4] | ((uint32_t)e2[5] << 16); pk2.w = e2[6] | ((uint32_t)e2[7] << 16);
+                }
+            }
+            *(u32x4*)&Bs[lr][ks] = pk;
+            if (DUAL) *(u32x4*)&B2s[lr][ks] = pk2;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK / 8; ++kk) {
+            const int kq = kk * 8 + (lane >> 5) * 4;
+            const bf16x4 av = *(const bf16x4*)&As[wm * 32 + (lane & 31)][kq];
+            const bf16x4 bv = *(const bf16x4*)&Bs[wn * 32 + (lane & 31)][kq];
+            acc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(av, bv, acc, 0, 0, 0);
+            if (DUAL) {
+                const bf16x4 b2 = *(const bf16x4*)&B2s[wn * 32 + (lane & 31)][kq];
+                acc2 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(av, b2, acc2, 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    const int n = t.n0 + wn * 32 + (lane & 31);
+    if (n >= a.N) return;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int r = wm * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+        if (r < t.rows) lg_store(a, t.p0 + r, n, acc[i], acc2[i], DUAL);
+    }
+}
+
+void launch_lgemm(const LGemmArgs& a, bool bf16, int groups, hipStream_t s) {
+    if (a.M <= 0 || a.N <= 0 || groups <= 0) return;
+    const dim3 grid((unsigned)((a.M + LG_BM - 1) / LG_BM), (unsigned)((a.N + LG_BN - 1) / LG_BN), (unsigned)groups);
+    if (bf16) {
+        if (a.W2) hipLaunchKernelGGL(lgemm_bf16_kernel<true>, grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(lgemm_bf16_kernel<false>, grid, dim3(256), 0, s, a);
+    } else {
+        if (a.W2) hipLaunchKernelGGL(lgemm_f32_kernel<true>, grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(lgemm_f32_kernel<false>, grid, dim3(256), 0, s, a);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// softmax attention whose values are its keys: paged key cache [n_pages][G][page][d]
+// ------------------------------------------------------------------------------------------------------------------
+template <int KVT>
+__global__ __launch_bounds__(256) void lay_k_append_kernel(const float* __restrict__ proj, int ldp, int k_off, void* __restrict__ kpool,
+                                                           const int32_t* __restrict__ bt, const LaySegDev* __restrict__ segs,
+                                                           const int32_t* __restrict__ rowseg, int G, int d, int page) {
+    const int r = blockIdx.x;
+    const LaySegDev sg = segs[rowseg[r]];
+    const int pos = sg.start_pos + (r - sg.row0);
+    const int pg = bt[sg.bt_off + pos / page];
+    const int n = G * d;
+    for (int i = threadIdx.x; i < n; i += 256) {
+        const int g = i / d, c = i - g * d;
+        const size_t dst = (((size_t)pg * G + g) * page + (size_t)(pos % page)) * d + c;
+        const float v = proj[(size_t)r * ldp + k_off + i];
+        if (KVT == KV_F32) ((float*)kpool)[dst] = v;
+        else ((uint16_t*)kpool)[dst] = f32_to_bf16(v);
+    }
+}
+void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int kvt, const int32_t* bt, const LaySegDev* segs,
+                         const int32_t* rowseg, int T, int G, int d, int page, hipStream_t s) {
+    if (T <= 0) return;
+    if (kvt == KV_F32) hipLaunchKernelGGL(lay_k_append_kernel<KV_F32>, dim3((unsigned)T), dim3(256), 0, s, proj, ldp, k_off, kpool, bt, segs, rowseg, G, d, page);
+    else hipLaunchKernelGGL(lay_k_append_kernel<KV_BF16>, dim3((unsigned)T), dim3(256), 0, s, proj, ldp, k_off, kpool, bt, segs, rowseg, G, d, page);
+}
+
+// A block = 16 query rows of one sequence and one key head: row qi = (position in the portion) * nrep + (query head in the
+// group), so that a single decode token fills the tile with the heads that share its keys.  16 lanes per query row.
+// Keys the tile can see: the kept first tokens [0, min(keep, lo)) and the window [lo, last position]; each query masks
+// with its own position.  Scores, softmax and the weighted sum are f32.
+constexpr int LA_BQ = 16;
+template <int KVT, int KT>
+__global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
+    extern __shared__ float lds[];
+    const int d = a.d, ldk = d + 1;
+    float* qs = lds;                       // [16][d]
+    float* ks = qs + LA_BQ * d;            // [KT][d + 1]
+    float* ps = ks + KT * ldk;             // [16][KT]
+    const int2 tile = a.tiles[blockIdx.x];
+    const LaySegDev sg = a.segs[tile.x];
+    const int g = blockIdx.y, nrep = a.H / a.G;
+    const int q0 = tile.y, nq = min(LA_BQ, sg.n * nrep - q0);
+    const int tid = threadIdx.x, qr = tid >> 4, ln = tid & 15;
+    const bool qvalid = qr < nq;
+    const int qi = q0 + (qvalid ? qr : 0);
+    const int lp = qi / nrep, head = g * nrep + (qi - lp * nrep);
+    const long long pos = (long long)sg.start_pos + lp;
+    const int row = sg.row0 + lp;
+    for (int i = ln; i < d; i += 16) qs[qr * d + i] = qvalid ? a.proj[(size_t)row * a.ldp + a.q_off + head * d + i] : 0.f;
+    const long long pmin = (long long)sg.start_pos + q0 / nrep, pmax = (long long)sg.start_pos + (q0 + nq - 1) / nrep;
+    const long long main_lo = max(0ll, pmin - a.win + 1);
+    const long long sink_hi = min(a.keep, main_lo);
+    const long long total = sink_hi + (pmax - main_lo + 1);
+    const float r1 = a.r1[head], r2 = a.r2[head];
+    float m = -INFINITY, l = 0.f, acc[16];
+#pragma unroll
+    for (int c = 0; c < 16; ++c) acc[c] = 0.f;
+    const size_t esz = KVT == KV_F32 ? 4 : 2;
+    for (long long v0 = 0; v0 < total; v0 += KT) {
+        __syncthreads();                   // previous tile fully consumed (and qs written, first time round)
+        for (int rr = 0; rr < KT / 16; ++rr) {
+            const int sl = qr + 16 * rr;
+            const long long v = v0 + sl;
+            if (v < total) {
+                const long long j = v < sink_hi ? v : main_lo + (v - sink_hi);
+                const int pg = a.bt[sg.bt_off + (int)(j / a.page)];
+                const char* src = (const char*)a.kpool + ((((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * d) * esz;
+                for (int i = ln; i < d; i += 16)
+                    ks[sl * ldk + i] = KVT == KV_F32 ? ((const float*)src)[i] : bf16_to_f32(((const uint16_t*)src)[i]);
+            } else {
+                for (int i = ln; i < d; i += 16) ks[sl * ldk + i] = 0.f;
+            }
+        }
+        __syncthreads();
+        float sc[KT / 16];
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int c = 0; c < KT / 16; ++c) {
+            const int sl = ln + 16 * c;
+            const long long v = v0 + sl;
+            const long long j = v < sink_hi ? v : main_lo + (v - sink_hi);
+            float dot = 0.f;
+            for (int i = 0; i < d; ++i) dot = fmaf(qs[qr * d + i], ks[sl * ldk + i], dot);
+            const long long dist = pos - j;
+            const bool vis = qvalid && v < total && dist >= 0 && (dist < a.win || j < a.keep);
+            sc[c] = vis ? dot * a.scale - r1 * log1pf(r2 * (float)dist) : -INFINITY;
+            tmax = fmaxf(tmax, sc[c]);
+        }
+        tmax = row16_max(tmax);
+        const float mn = fmaxf(m, tmax);
+        const float corr = mn == -INFINITY ? 1.f : expf(m - mn);     // m = -inf, mn finite: exp(-inf) = 0
+        float psum = 0.f;
+#pragma unroll
+        for (int c = 0; c < KT / 16; ++c) {
+            const float p = sc[c] == -INFINITY ? 0.f : expf(sc[c] - mn);
+            ps[qr * KT + ln + 16 * c] = p;
+            psum += p;
+        }
+        psum = row16_sum(psum);
+        l = l * corr + psum;
+        m = mn;
+        __syncthreads();
+        const int kn = (int)min((long long)KT, total - v0);
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const int i = ln + 16 * c;
+            if (i < d) {
+                float o = acc[c] * corr;
+                for (int sl = 0; sl < kn; ++sl) o = fmaf(ps[qr * KT + sl], ks[sl * ldk + i], o);
+                acc[c] = o;
+            }
+        }
+    }
+    if (!qvalid) return;
+    const float gate = a.proj[(size_t)row * a.ldp + a.g_off + head];
+    const float inv = gate / l;
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+        const int i = ln + 16 * c;
+        if (i < d) a.out[(size_t)row * a.ldo + head * d + i] = acc[c] * inv;
+    }
+}
+void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s) {
+    if (a.ntiles <= 0) return;
+    const dim3 grid((unsigned)a.ntiles, (unsigned)a.G);
+    const bool narrow = a.d > 128;         // 32-key tiles keep the block inside 64 KiB of LDS up to d = 256
+    const int KT = narrow ? 32 : 64;
+    const size_t lds = (size_t)(LA_BQ * a.d + KT * (a.d + 1) + LA_BQ * KT) * sizeof(float);
+    if (kvt == KV_F32) {
+        if (narrow) hipLaunchKernelGGL((lay_attn_kernel<KV_F32, 32>), grid, dim3(256), lds, s, a);
+        else hipLaunchKernelGGL((lay_attn_kernel<KV_F32, 64>), grid, dim3(256), lds, s, a);
+    } else {
+        if (narrow) hipLaunchKernelGGL((lay_attn_kernel<KV_BF16, 32>), grid, dim3(256), lds, s, a);
+        else hipLaunchKernelGGL((lay_attn_kernel<KV_BF16, 64>), grid, dim3(256), lds, s, a);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// lightning attention: S_t = decay S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, per head, state [d][e] f32 per sequence.
+// A block owns one (sequence, head, slice of ES value columns) and walks the portion in chunks of C tokens:
+//   o_t = decay^(t+1) S0^T q_t + sum_(s <= t) decay^(t-s) (q_t . k_s) v_s,   S <- decay^n S0 + sum_s decay^(n-1-s) k_s v_s^T
+// (t, s local to the chunk of n tokens).  Everything is f32.
+// ------------------------------------------------------------------------------------------------------------------
+constexpr int LL_ES = 32;
+__global__ __launch_bounds__(256) void lay_lightning_kernel(LLightArgs a, int C) {
+    extern __shared__ float lds[];
+    const int d = a.d, e = a.e;
+    float* S = lds;                        // [d][ES]
+    float* qs = S + d * LL_ES;             // [C][d]
+    float* ks = qs + C * d;                // [C][d]
+    float* vs = ks + C * d;                // [C][ES]
+    float* As = vs + C * LL_ES;            // [C][C]
+    float* pw = As + C * C;                // [C + 1] decay^n
+    const LaySegDev sg = a.segs[blockIdx.x];
+    const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
+    const int ne = min(LL_ES, e - j0);
+    const float decay = a.decay[head];
+    float* st = a.state_pool + (size_t)sg.slot * a.slot_stride + a.st_off + (size_t)head * d * e;
+    for (int idx = tid; idx < d * LL_ES; idx += 256) {
+        const int i = idx / LL_ES, j = idx % LL_ES;
+        S[idx] = j < ne ? st[(size_t)i * e + j0 + j] : 0.f;
+    }
+    if (tid <= C) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
+    for (int t0 = 0; t0 < sg.n; t0 += C) {
+        const int n = min(C, sg.n - t0);
+        __syncthreads();                   // S, pw ready; the previous chunk's q / k / v no longer read
+        for (int idx = tid; idx < n * d; idx += 256) {
+            const int t = idx / d, i = idx - t * d;
+            const size_t base = (size_t)(sg.row0 + t0 + t) * a.ldp + (size_t)head * d + i;
+            qs[idx] = a.proj[base + a.q_off];
+            ks[idx] = a.proj[base + a.k_off];
+        }
+        for (int idx = tid; idx < n * LL_ES; idx += 256) {
+            const int t = idx / LL_ES, j = idx % LL_ES;
+            vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + t0 + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < n * n; idx += 256) {
+            const int t = idx / n, s = idx - t * n;
+            float dot = 0.f;
+            if (s <= t) {
+                for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * d + i], dot);
+                dot *= pw[t - s];
+            }
+            As[t * C + s] = dot;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < n * LL_ES; idx += 256) {
+            const int t = idx / LL_ES, j = idx % LL_ES;
+            float inter = 0.f;
+            for (int i = 0; i < d; ++i) inter = fmaf(S[i * LL_ES + j], qs[t * d + i], inter);
+            float o = inter * pw[t + 1];
+            for (int s = 0; s <= t; ++s) o = fmaf(As[t * C + s], vs[s * LL_ES + j], o);
+            if (j < ne) a.out[(size_t)(sg.row0 + t0 + t) * a.ldo + (size_t)head * e + j0 + j] = o;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < d * LL_ES; idx += 256) {
+            const int i = idx / LL_ES, j = idx % LL_ES;
+            float sv = S[idx] * pw[n];
+            for (int s = 0; s < n; ++s) sv = fmaf(pw[n - 1 - s] * ks[s * d + i], vs[s * LL_ES + j], sv);
+            S[idx] = sv;
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < d * LL_ES; idx += 256) {
+        const int i = idx / LL_ES, j = idx % LL_ES;
+        if (j < ne) st[(size_t)i * e + j0 + j] = S[idx];
+    }
+}
+void launch_lay_lightning(const LLightArgs& a, hipStream_t s) {
+    if (a.nseg <= 0) return;
+    const int C = a.d > 128 ? 8 : 16;
+    const size_t lds = (size_t)(a.d * LL_ES + 2 * C * a.d + C * LL_ES + C * C + C + 1) * sizeof(float);
+    hipLaunchKernelGGL(lay_lightning_kernel, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES)), dim3(256), lds, s, a, C);
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// mixture of experts: router + counting sort
+// ------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void lay_router_kernel(const float* __restrict__ h, const uint16_t* __restrict__ wr, int32_t* __restrict__ sel,
+                                                         float* __restrict__ wsel, int W, int E, int top) {
+    extern __shared__ float zs[];          // [E]
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float* hr = h + (size_t)t * W;
+    for (int ex = wave; ex < E; ex += 4) {
+        float s = 0.f;
+        for (int i = lane; i < W; i += 64) s = fmaf(hr[i], bf16_to_f32(wr[(size_t)ex * W + i]), s);
+        s = wave_sum(s);
+        if (lane == 0) zs[ex] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 0; k < top; ++k) {
+            int best = -1; float bz = 0.f;
+            for (int ex = 0; ex < E; ++ex) {
+                const float z = zs[ex];
+                if (z == -INFINITY) continue;
+                if (best < 0 || z > bz) { best = ex; bz = z; }
+            }
+            if (best < 0) { best = 0; bz = 0.f; }
+            sel[(size_t)t * top + k] = best;
+            wsel[(size_t)t * top + k] = 1.f / (1.f + expf(-bz));
+            zs[best] = -INFINITY;
+        }
+    }
+}
+void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s) {
+    if (T <= 0) return;
+    hipLaunchKernelGGL(lay_router_kernel, dim3((unsigned)T), dim3(256), (size_t)E * sizeof(float), s, h, wr, sel, wsel, W, E, top);
+}
+
+__global__ __launch_bounds__(1024) void lay_moe_plan_kernel(const int32_t* __restrict__ sel, int32_t* __restrict__ off, int32_t* __restrict__ srt,
+                                                            int n, int E) {
+    extern __shared__ int cnt[];           // [E] counts, then cursors
+    for (int i = threadIdx.x; i < E; i += 1024) cnt[i] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n; p += 1024) atomicAdd(&cnt[sel[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int i = 0; i < E; ++i) { const int c = cnt[i]; off[i] = run; cnt[i] = run; run += c; }
+        off[E] = run;
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < n; p += 1024) srt[atomicAdd(&cnt[sel[p]], 1)] = p;
+}
+void launch_lay_moe_plan(const int32_t* sel, int32_t* off, int32_t* srt, int n, int E, hipStream_t s) {
+    hipLaunchKernelGGL(lay_moe_plan_kernel, dim3(1), dim3(1024), (size_t)E * sizeof(int), s, sel, off, srt, n, E);
+}
+
+// arg-max of every row, lowest index among equals
+__global__ __launch_bounds__(256) void lay_argmax_rows_kernel(const float* __restrict__ logits, int ld, int V, uint32_t* __restrict__ out) {
+    __shared__ float bv[256];
+    __shared__ int bi[256];
+    const float* lr = logits + (size_t)blockIdx.x * ld;
+    float best = -INFINITY; int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += 256) { const float v = lr[i]; if (v > best) { best = v; idx = i; } }
+    bv[threadIdx.x] = best; bi[threadIdx.x] = idx;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) {
+        if ((int)threadIdx.x < st) {
+            const float ov = bv[threadIdx.x + st]; const int oi = bi[threadIdx.x + st];
+            if (ov > bv[threadIdx.x] || (ov == bv[threadIdx.x] && oi < bi[threadIdx.x])) { bv[threadIdx.x] = ov; bi[threadIdx.x] = oi; }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = (uint32_t)(bi[0] == 0x7fffffff ? 0 : bi[0]);
+}
+void launch_lay_argmax_rows(const float* logits, int ld, int V, uint32_t* out, int n_rows, hipStream_t s) {
+    if (n_rows <= 0) return;
+    hipLaunchKernelGGL(lay_argmax_rows_kernel, dim3((unsigned)n_rows), dim3(256), 0, s, logits, ld, V, out);
+}
+
+}  // namespace cm

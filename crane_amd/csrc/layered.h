@@ -1,0 +1,114 @@
+// Layer-list decoders: a model whose config.json spells out every layer (mixer kind + sizes, feed-forward kind + sizes) instead
+// of a family-wide geometry.  First member: Korupel (sandwich RMS norms with a scaled residual, a short causal convolution in front
+// of every sublayer, softmax attention over a sliding window with kept first tokens / a logarithmic distance penalty / values that
+// are the keys / one sigmoid gate per head, lightning (decayed linear) attention, dense GELU or sigmoid-routed mixture-of-experts
+// feed-forwards).  The mechanisms are kernels with their constants as arguments (kernels_layered.hip); the per-layer plumbing and
+// the step function over mixed batches (prompt portions beside single decode tokens) are in model_layered.cpp.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+namespace cm {
+
+enum { LMIX_ATTN = 0, LMIX_LIGHTNING = 1 };
+enum { LMLP_NONE = 0, LMLP_DENSE = 1, LMLP_MOE = 2 };
+enum { LACT_NONE = 0, LACT_SILU = 1, LACT_SIGMOID = 2, LACT_GELU_TANH = 3 };
+
+// one entry of config "layers"
+struct LayerSpec {
+    int mixer = LMIX_ATTN;
+    int heads = 0, kv_heads = 0, dim = 0, vdim = 0;
+    float scale = 1.f;                 // attention: score multiplier
+    long long win = 0, keep = 0;       // attention: window size, kept first tokens
+    std::vector<float> decay;          // lightning: per head
+    int mlp = LMLP_NONE, ff = 0, experts = 0, top = 0;
+};
+
+// device-side weights of one layer (bf16 matrices [out, in], f32 vectors)
+struct LayeredLayerW {
+    float *norm1 = nullptr, *norm1b = nullptr, *norm2 = nullptr, *norm2b = nullptr;
+    float *canon1 = nullptr, *canon2 = nullptr;      // [W][taps]
+    // mixer input projection, rows concatenated so that one GEMM produces them:
+    //   attention: q (H d) | k (G d) | g (H);  lightning: q (H d) | k (H d) | v (H e) | g (H e)
+    uint16_t* in_w = nullptr;
+    float* in_b = nullptr;                           // [rows] (zeros where the checkpoint has no bias) or null
+    int in_rows = 0, q_off = 0, k_off = 0, v_off = 0, g_off = 0;
+    uint16_t* o_w = nullptr;                         // [W][H e]
+    float *r1 = nullptr, *r2 = nullptr;              // attention: per-head distance penalty
+    float* decay = nullptr;                          // lightning: per head
+    float* mix_norm = nullptr;                       // lightning: [H e]
+    uint16_t *gate = nullptr, *up = nullptr, *down = nullptr;   // dense: [ff][W], [ff][W], [W][ff]; experts: [E] of each, back to back
+    uint16_t* router = nullptr;                      // [E][W]
+    int kv_idx = -1;                                 // index among the attention layers
+    size_t k_pool_off = 0, k_page_bytes = 0;         // this layer's key pages inside the pool
+    size_t st_off = 0;                               // lightning state offset inside a slot of the state pool (floats)
+    size_t c1_off = 0, c2_off = 0;                   // convolution tails inside a slot of the conv pool (floats)
+};
+
+// rows [row0, row0 + n) of a pass are positions start_pos.. of the sequence in `slot`; its page table starts at bt_off
+struct LaySegDev { int row0, n, start_pos, slot, bt_off, pad0, pad1, pad2; };
+
+struct LGemmArgs {
+    const float* A = nullptr; int lda = 0;
+    const int32_t* a_idx = nullptr; int a_div = 1;   // A row of output row p: a_idx ? a_idx[p] / a_div : p
+    const uint16_t* W = nullptr;                     // [N][K] bf16
+    const uint16_t* W2 = nullptr;                    // second matrix: C = act(A W^T) * (A W2^T)
+    size_t w_stride = 0;                             // elements between the matrices of consecutive groups
+    const float* bias = nullptr;                     // [N] or null
+    float* C = nullptr; int ldc = 0;
+    const int32_t* c_idx = nullptr;                  // output row of p: c_idx ? c_idx[p] : p
+    int M = 0, N = 0, K = 0;
+    const int32_t* grp_off = nullptr;                // grouped: rows [grp_off[g], grp_off[g + 1]) use matrix g; M bounds a group's rows
+    int act = LACT_NONE, act2 = LACT_NONE, act_split = 0;   // columns < act_split: act, the others act2 (W2: act on the first product)
+};
+// bf16 = true: A rounded to bfloat16, matrix cores, f32 accumulation; false: f32 FMA throughout
+void launch_lgemm(const LGemmArgs& a, bool bf16, int groups, hipStream_t s);
+
+void launch_lay_rms_rows(const float* x, const int32_t* rows, const float* w, float* out, int n_rows, int W, float eps, hipStream_t s);
+// out = h + conv(h) over time per channel; the taps - 1 inputs before a portion come from the sequence's tail in conv_pool
+void launch_lay_canon(const float* h, float* out, const float* cw, const float* conv_pool, size_t slot_stride, size_t off,
+                      const LaySegDev* segs, const int32_t* rowseg, int T, int W, int taps, hipStream_t s);
+void launch_lay_canon_tail(const float* h, float* conv_pool, size_t slot_stride, size_t off, const LaySegDev* segs, int nseg, int W,
+                           int taps, hipStream_t s);
+// single-token rows only (every segment n = 1): RMS norm, convolution and tail shift in one launch
+void launch_lay_norm_canon_decode(const float* x, const float* nw, float eps, float* out, const float* cw, float* conv_pool,
+                                  size_t slot_stride, size_t off, const LaySegDev* segs, int T, int W, int taps, hipStream_t s);
+// x += mult * RMSNorm(y) * w;  sel != null: y[r] = sum_k wsel[r top + k] * ys[r top + k] (mixture-of-experts combine)
+void launch_lay_post_norm(float* x, const float* y, const float* w, float mult, float eps, int T, int W, const float* wsel, int top,
+                          hipStream_t s);
+
+struct LAttnArgs {
+    const float* proj; int ldp, q_off, g_off;        // activated projection rows: q | k | gate
+    float* out; int ldo;                             // [T][H d], gated
+    const void* kpool;                               // [n_pages][G][page][d]
+    const int32_t* bt; const LaySegDev* segs; const int2* tiles; int ntiles;
+    const float *r1, *r2;
+    int H, G, d, page;
+    float scale; long long win, keep;
+};
+void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int kvt, const int32_t* bt, const LaySegDev* segs,
+                         const int32_t* rowseg, int T, int G, int d, int page, hipStream_t s);
+void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s);    // kvt: KV_BF16 | KV_F32
+
+struct LLightArgs {
+    const float* proj; int ldp, q_off, k_off, v_off; // activated projection rows
+    float* out; int ldo;                             // [T][H e] before the norm
+    float* state_pool; size_t slot_stride, st_off;   // [slot] ... [H][d][e] f32
+    const LaySegDev* segs; int nseg;
+    const float* decay;
+    int H, d, e;
+};
+void launch_lay_lightning(const LLightArgs& a, hipStream_t s);
+// out = o / rms(o) * w * gate over whole rows (gate already passed through the sigmoid)
+void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s);
+
+// router: z = h . Wr^T in f32, the `top` largest (lowest index first among equals) -> sel [T top], wsel = sigmoid(z)
+void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s);
+// counting sort of the T top (token, choice) pairs by expert: off [E + 1], srt [T top]
+void launch_lay_moe_plan(const int32_t* sel, int32_t* off, int32_t* srt, int n, int E, hipStream_t s);
+void launch_lay_argmax_rows(const float* logits, int ld, int V, uint32_t* out, int n_rows, hipStream_t s);
+
+}  // namespace cm

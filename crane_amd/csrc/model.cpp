@@ -106,6 +106,11 @@ void Model::init_common(const std::string& config_json, const cm_opts* o) {
     const cmjson::Value* root = j.get();
     // VLM checkpoints nest the LM config under text_config
     if (root->has("text_config") && !root->has("hidden_size")) root = root->get("text_config");
+    // model registry: a config with "architecture" and a "layers" list is a layer-list decoder (model_layered.cpp); everything
+    // else is the Qwen3 / Qwen3.5 geometry keyed by "model_type"
+    const bool is_layered = root->get("architecture") != nullptr && root->get("layers") != nullptr;
+    if (is_layered) init_layered_config(*root);
+    else {
     cfg.model_type = root->string("model_type", j->string("model_type", "qwen3"));
     cfg.V = (int)root->integer("vocab_size", 0);
     cfg.H = (int)root->integer("hidden_size", 0);
@@ -221,6 +226,7 @@ void Model::init_common(const std::string& config_json, const cm_opts* o) {
     if (cfg.D != 128 && cfg.D != 256) throw CmError(CM_ERR_UNSUPPORTED, "head_dim must be 128 or 256");
     if (cfg.H % 8 || cfg.I % 8) throw CmError(CM_ERR_UNSUPPORTED, "hidden/intermediate must be multiples of 8");
     if (cfg.Hq % cfg.Hkv) throw CmError(CM_ERR_INVALID, "num_attention_heads % num_key_value_heads != 0");
+    }
 
     dev = opts.device;
     if (!plan_only) {
@@ -298,6 +304,7 @@ void Model::init_common(const std::string& config_json, const cm_opts* o) {
 }
 
 void Model::alloc_runtime() {
+    if (layered) { alloc_runtime_layered(); return; }
     const int H = cfg.H, D = cfg.D;
     x = dalloc<float>(H);
     y = dalloc<float>(H);
@@ -702,10 +709,10 @@ int Model::seq_alloc() {
 void Model::seq_truncate(int s, size_t new_len) {
     Seq& q = seq(s);
     if ((int64_t)new_len > q.len) throw CmError(CM_ERR_RANGE, "truncate beyond cached length");
-    if (gdn_layers > 0 && (int64_t)new_len != q.len) {
-        // a recurrent (GDN) state cannot be rewound: only "clear" is possible, like the reference,
-        // which re-prefills from scratch after preemption (engine/mod.rs:430-504)
-        if (new_len != 0) throw CmError(CM_ERR_UNSUPPORTED, "Gated-Delta-Net state cannot be truncated to a non-zero length");
+    if ((conv_pool || state_pool) && (int64_t)new_len != q.len) {
+        // a recurrent state (GDN, lightning attention, convolution tails) cannot be rewound: only "clear" is possible, like the
+        // reference, which re-prefills from scratch after preemption (engine/mod.rs:430-504)
+        if (new_len != 0) throw CmError(CM_ERR_UNSUPPORTED, "a recurrent state cannot be truncated to a non-zero length");
         reset_gdn_state(s);
     }
     // a sequence cut back INTO an image prompt would rotate its next tokens at cache position + rope_delta < 0
@@ -723,9 +730,8 @@ void Model::seq_truncate(int s, size_t new_len) {
 }
 
 void Model::reset_gdn_state(int slot) {
-    if (gdn_layers == 0) return;
-    CM_HIP(hipMemsetAsync(conv_pool + conv_slot_elems * (size_t)slot, 0, conv_slot_elems * sizeof(float), stream));
-    CM_HIP(hipMemsetAsync(state_pool + state_slot_elems * (size_t)slot, 0, state_slot_elems * sizeof(float), stream));
+    if (conv_pool) CM_HIP(hipMemsetAsync(conv_pool + conv_slot_elems * (size_t)slot, 0, conv_slot_elems * sizeof(float), stream));
+    if (state_pool) CM_HIP(hipMemsetAsync(state_pool + state_slot_elems * (size_t)slot, 0, state_slot_elems * sizeof(float), stream));
 }
 
 void Model::seq_free(int s) {
@@ -743,12 +749,11 @@ int Model::seq_fork(int src) {
     b.rope_delta = a.rope_delta;
     b.pages = a.pages;
     for (int32_t p : b.pages) page_ref[(size_t)p]++;
-    if (gdn_layers > 0) {      // recurrent + conv state travel with the sequence
-        CM_HIP(hipMemcpyAsync(conv_pool + conv_slot_elems * (size_t)d, conv_pool + conv_slot_elems * (size_t)src,
-                              conv_slot_elems * sizeof(float), hipMemcpyDeviceToDevice, stream));
-        CM_HIP(hipMemcpyAsync(state_pool + state_slot_elems * (size_t)d, state_pool + state_slot_elems * (size_t)src,
-                              state_slot_elems * sizeof(float), hipMemcpyDeviceToDevice, stream));
-    }
+    // recurrent + conv state travel with the sequence
+    if (conv_pool) CM_HIP(hipMemcpyAsync(conv_pool + conv_slot_elems * (size_t)d, conv_pool + conv_slot_elems * (size_t)src,
+                                         conv_slot_elems * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    if (state_pool) CM_HIP(hipMemcpyAsync(state_pool + state_slot_elems * (size_t)d, state_pool + state_slot_elems * (size_t)src,
+                                          state_slot_elems * sizeof(float), hipMemcpyDeviceToDevice, stream));
     // copy-on-write of the last, partially filled page: both forks will append into it
     if (!b.pages.empty() && (a.len % page) != 0) {
         if (free_pages.empty()) { seq_free(d); throw CmError(CM_ERR_OOM, "KV pool exhausted"); }
@@ -768,6 +773,7 @@ void Model::cow_page(int s, size_t idx) {
     page_ref[(size_t)newp] = 1;
     page_ref[(size_t)oldp]--;
     q.pages[idx] = newp;
+    if (layered) { layered_cow_page(oldp, newp); if (active_seq == s) active_pages_uploaded = std::min(active_pages_uploaded, idx); return; }
     const size_t pitch = (size_t)n_pages * page_bytes;
     CM_HIP(hipMemcpy2DAsync(kv_pool + (size_t)newp * page_bytes, pitch, kv_pool + (size_t)oldp * page_bytes, pitch,
                             page_bytes, (size_t)n_kv_layers * 2, hipMemcpyDeviceToDevice, stream));
@@ -812,10 +818,12 @@ void Model::activate(int s) {
 uint64_t Model::kv_bytes() const {
     uint64_t pages_used = 0;
     for (auto r : page_ref) if (r > 0) ++pages_used;
+    if (layered) return pages_used * page_bytes;      // page_bytes: every attention layer's share of one page (keys only)
     return pages_used * page_bytes * 2ull * (uint64_t)n_kv_layers;
 }
 
 uint64_t Model::decode_bytes_per_token(size_t ctx) const {
+    if (layered) return layered_decode_bytes(ctx);
     // 2 B x every weight element once + KV read at ctx (+ GDN state read+write), this rank
     const uint64_t H = cfg.H, D = cfg.D;
     const uint64_t mlp = 3ull * I_l * H + 2 * H;
@@ -1135,7 +1143,7 @@ int Model::prefill_chunk_rows() const {
 }
 
 void Model::ensure_prefill_buffers() {
-    if (pX) return;
+    if (pX || layered) return;
     const int H = cfg.H, D = cfg.D;
     chunk = prefill_chunk_rows();
     chunk_pad = (chunk + 127) / 128 * 128;
@@ -1486,6 +1494,12 @@ void Model::prefill_layers(int S, const PrefillSeg* segs, int nseg, size_t off) 
 // gives: its K/V pages (and GDN state), the arg-max of its last position in greedy_out[i], its logits in logitsb[i * V].
 void Model::prefill_multi(const int32_t* sq, const uint32_t* const* ids, const size_t* lens, size_t n_items, uint32_t* greedy_out) {
     if (n_items == 0 || n_items > (size_t)MAXB) throw CmError(CM_ERR_INVALID, "prefill_multi: 1..128 sequences");
+    if (layered) {                                               // whole prompts from position 0 = one step of fresh sequences
+        std::vector<StepItem> it(n_items);
+        for (size_t i = 0; i < n_items; ++i) { seq_truncate(sq[i], 0); it[i] = StepItem{sq[i], ids[i], lens[i], nullptr, -1}; }
+        step_batch(it.data(), n_items, nullptr, greedy_out);
+        return;
+    }
     if (kvq()) throw CmError(CM_ERR_UNSUPPORTED, "prefill_multi over quantised KV pages");
     if (rccl && cfg.V % tp != 0) throw CmError(CM_ERR_UNSUPPORTED, "prefill_multi under tensor parallelism needs vocab_size divisible by tp_size");
     ensure_prefill_buffers();
@@ -1710,7 +1724,7 @@ void Model::lm_head_rows(int nb, bool want_rows) {
 // masks or KV copies -- up to MAXB sequences share ONE pass over the weights
 // ------------------------------------------------------------------------------------
 void Model::ensure_batch_buffers() {
-    if (stb) return;
+    if (stb || layered) return;
     const int H = cfg.H, D = cfg.D;
     const size_t attn_rows = (size_t)(cfg.hybrid ? 2 * Hq_l + 2 * Hkv_l : Hq_l + 2 * Hkv_l) * D;
     ldq = (int)std::max(attn_rows, (size_t)in_proj_pad);
@@ -1751,6 +1765,14 @@ void Model::ensure_batch_buffers() {
 
 void Model::decode_batch(const int32_t* sq, const uint32_t* toks, size_t n, float* logits_out, uint32_t* greedy_out,
                          const std::function<void(size_t, int)>* after_group) {
+    if (layered) {                                          // one token per sequence = one step of single-token items
+        if (n == 0 || n > (size_t)MAXB) throw CmError(CM_ERR_INVALID, "decode_batch: 1..128 sequences");
+        std::vector<StepItem> it(n);
+        for (size_t i = 0; i < n; ++i) it[i] = StepItem{sq[i], toks + i, 1, nullptr, -1};
+        step_batch(it.data(), n, logits_out, greedy_out);
+        if (after_group) (*after_group)(0, (int)n);
+        return;
+    }
     if (rccl && cfg.V % tp != 0) throw CmError(CM_ERR_UNSUPPORTED, "batched decode under tensor parallelism needs vocab_size divisible by tp_size");
     if (quantized && !quant_act_int)
         throw CmError(CM_ERR_UNSUPPORTED, "batched decode over quantised weights needs the integer-dot activation mode (CM_QUANT_ACT unset)");
@@ -2068,6 +2090,7 @@ void Model::decode_batch(const int32_t* sq, const uint32_t* toks, size_t n, floa
 // ------------------------------------------------------------------------------------
 void Model::forward(int s, const uint32_t* ids, size_t n, size_t start_pos, float* logits_out, uint32_t* greedy_out) {
     if (n == 0 || ids == nullptr) throw CmError(CM_ERR_INVALID, "empty input");
+    if (layered) { layered_forward(s, ids, n, start_pos, logits_out, greedy_out); return; }
     Seq& q = seq(s);
     if ((int64_t)start_pos > q.len) throw CmError(CM_ERR_RANGE, "start_pos beyond cached length");
     if (start_pos + n > (size_t)max_seq) throw CmError(CM_ERR_RANGE, "start_pos + n exceeds max_seq_len");
@@ -2172,6 +2195,12 @@ void Model::generate(const uint32_t* prompt, size_t n_prompt, const cm_gen_confi
         if (cb && cb(user, t) != 0) stop = true;
     };
     emit(tok);
+    if (layered && !device_pick) {                          // greedy: the arg-max row of each step
+        while (!stop && produced < g.max_new_tokens) {
+            forward(0, &out[n - 1], 1, n - 1, nullptr, &tok);
+            emit(tok);
+        }
+    } else
     if (device_pick) {
         while (!stop && produced < g.max_new_tokens) {
             forward(0, &out[n - 1], 1, n - 1, nullptr, nullptr);
@@ -2203,6 +2232,19 @@ void Model::generate(const uint32_t* prompt, size_t n_prompt, const cm_gen_confi
 }
 
 void Model::bench_decode(uint32_t first, size_t k, uint32_t* toks, float* ms) {
+    if (layered) {                                          // k greedy steps of sequence 0 through the step function
+        if (k == 0) throw CmError(CM_ERR_INVALID, "k must be positive");
+        hipEvent_t e0, e1;
+        CM_HIP(hipEventCreate(&e0)); CM_HIP(hipEventCreate(&e1));
+        uint32_t t = first;
+        CM_HIP(hipEventRecord(e0, stream));
+        for (size_t i = 0; i < k; ++i) { forward(0, &t, 1, (size_t)seq(0).len, nullptr, &t); if (toks) toks[i] = t; }
+        CM_HIP(hipEventRecord(e1, stream));
+        CM_HIP(hipEventSynchronize(e1));
+        if (ms) CM_HIP(hipEventElapsedTime(ms, e0, e1));
+        (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+        return;
+    }
     if (k == 0 || k > (size_t)RING) throw CmError(CM_ERR_INVALID, "k must be in 1..4096");
     Seq& q = seq(0);
     ensure_pages(0, q.len + (int64_t)k);
@@ -2231,6 +2273,7 @@ void Model::bench_decode(uint32_t first, size_t k, uint32_t* toks, float* ms) {
 
 void Model::bench_kernel(const std::string& which, size_t iters, float* ms, uint64_t* bytes) {
     if (iters == 0) throw CmError(CM_ERR_INVALID, "iters == 0");
+    if (layered) throw CmError(CM_ERR_UNSUPPORTED, "bench_kernel: not available for layer-list decoders");
     const int H = cfg.H, D = cfg.D;
     const int v_eff = std::max(0, std::min(V_l, cfg.V - v0));
     uint64_t b = 0;
@@ -2435,6 +2478,7 @@ void Model::debug_qgemv(int layer, const std::string& which, const float* xh, si
 }
 
 void Model::debug_fill_kv(size_t ctx, uint64_t seed) {
+    if (layered) throw CmError(CM_ERR_UNSUPPORTED, "debug_fill_kv: not available for layer-list decoders");
     seq_truncate(0, 0);
     ensure_pages(0, (int64_t)ctx);
     activate(0);

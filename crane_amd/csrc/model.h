@@ -12,6 +12,9 @@
 
 #include "../../include/crane_mi355.h"
 #include "kernels.h"
+#include "layered.h"
+
+namespace cmjson { struct Value; }
 
 namespace cm {
 
@@ -116,6 +119,9 @@ struct VisionW {
     struct Merger { float *n_w = nullptr, *n_b = nullptr, *fc1_b = nullptr, *fc2_b = nullptr; uint16_t *fc1_w = nullptr, *fc2_w = nullptr; };
     std::vector<Merger> deep;     // deepstack_merger_list.k: LayerNorm over the regrouped 4 x hidden row, fc1 + GELU, fc2
 };
+
+struct Layered;      // layer-list decoders: specs, weights and pass scratch (model_layered.cpp)
+struct LayeredDeleter { void operator()(Layered* p) const; };
 
 struct Rccl;         // dlopen'ed RCCL entry points + communicator, or the peer-store transport of an in-process group (tp.cpp)
 struct PeerShared;   // state shared by the ranks of an in-process tensor-parallel group (tp.h)
@@ -404,6 +410,23 @@ int prefill_lo_mask = 0;              // EXPERIMENT (cm_debug_set "prefill_lo_ma
 
     ~Model();
 
+    // ---- layer-list decoders (layered.h, model_layered.cpp): config "architecture" + "layers" instead of a family geometry ----
+    bool layered = false;
+    std::unique_ptr<Layered, LayeredDeleter> lay;
+    // one request's share of a step: its next n tokens (continuing at the sequence's cached length) and the positions among them
+    // whose logits are wanted (ascending; n_want < 0: the last one)
+    struct StepItem { int32_t seq; const uint32_t* ids; size_t n; const int32_t* want; int32_t n_want; };
+    // all items as ONE batch -- prompt portions beside single decode tokens; logits_out [wanted rows][V] and greedy_out [wanted rows]
+    // in the order of the items and their wanted positions (either may be null)
+    void step_batch(const StepItem* items, size_t n_items, float* logits_out, uint32_t* greedy_out);
+    void init_layered_config(const cmjson::Value& root);
+    void alloc_runtime_layered();
+    void layered_forward(int s, const uint32_t* ids, size_t n, size_t start_pos, float* logits_out, uint32_t* greedy_out);
+    void layered_cow_page(int32_t oldp, int32_t newp);
+    uint64_t layered_decode_bytes(size_t ctx) const;
+    void layered_set_capture(bool on);                    // cm_debug_set("lay_capture")
+    size_t layered_capture(float* out, size_t n) const;   // cm_debug_read("lay_layers"): [pass][layer][row][width]; returns the count
+
     // ---- construction ----
     void init_common(const std::string& config_json, const cm_opts* o);
     void alloc_runtime();
@@ -450,6 +473,8 @@ int prefill_lo_mask = 0;              // EXPERIMENT (cm_debug_set "prefill_lo_ma
 // loaders (loader.cpp)
 void load_from_dir(Model& m, const std::string& dir);
 void load_synthetic(Model& m, uint64_t seed);
+void load_layered_from_dir(Model& m, const std::string& dir);      // model_layered.cpp
+void load_layered_synthetic(Model& m, uint64_t seed);
 std::string tp_shard_plan_json(const std::string& config_json, int tp_size, int tp_rank);   // loader.cpp, host only
 std::string gguf_config_json(const std::string& path);     // loader_gguf.cpp
 void load_from_gguf(Model& m, const std::string& path);

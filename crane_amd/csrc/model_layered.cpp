@@ -1,0 +1,625 @@
+// Layer-list decoders on the Model runtime (layered.h): configuration, weights, per-sequence state and the step function.
+//
+// What is shared with the other families: the handle and its options, the sequence table and the page allocator (Seq, ensure_pages,
+// seq_alloc / seq_free / seq_fork / seq_truncate), the per-slot state pools (conv_pool: the convolution tails of every sublayer,
+// state_pool: the linear-attention states), the embedding gather, the logits rows the samplers read (logitsb), the engine.
+// What is new: Model::step_batch -- ONE pass over the weights for any mix of prompt portions and single decode tokens, each
+// continuing its sequence from the cache and state earlier steps left; forward / prefill_multi / decode_batch / generate and the
+// engine's scheduler all go through it for this family.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <map>
+
+#include "json_min.h"
+#include "model.h"
+#include "safetensors.h"
+
+namespace cm {
+
+struct Layered {
+    std::vector<LayerSpec> spec;
+    std::vector<LayeredLayerW> w;
+    int taps = 0;                      // 0: no convolution in front of the sublayers
+    float mult = 1.f;
+    bool f32 = false;                  // number format of the projections and the key cache
+    float* final_norm = nullptr;
+    uint16_t* head = nullptr;
+    int cap = 0;                       // rows of one pass
+    int max_in = 0, max_o = 0, max_ff = 0, max_top = 1, max_E = 1;
+    std::vector<int> nreps;            // distinct query-heads-per-key-head values of the attention layers
+    float *X = nullptr, *Hn = nullptr, *Hc = nullptr, *P = nullptr, *O = nullptr, *O2 = nullptr, *Y = nullptr, *HH = nullptr, *YS = nullptr,
+          *wsel = nullptr, *Xw = nullptr;
+    int32_t *sel = nullptr, *srt = nullptr, *off = nullptr;
+    uint32_t *d_greedy = nullptr, *h_greedy = nullptr;
+    float* h_rows = nullptr;           // pinned staging of logits rows
+    int32_t *d_tab = nullptr, *h_tab = nullptr;
+    size_t tab_ints = 0;
+    static constexpr int LOGIT_ROWS = 256;
+    bool capture = false;              // cm_debug_set("lay_capture"): keep the residual stream after every layer of every pass
+    std::vector<float> captured;
+    ~Layered() {
+        if (h_greedy) (void)hipHostFree(h_greedy);
+        if (h_rows) (void)hipHostFree(h_rows);
+        if (h_tab) (void)hipHostFree(h_tab);
+    }
+};
+
+void LayeredDeleter::operator()(Layered* p) const { delete p; }
+
+static int act_of(const std::string& s) { return s == "attention" ? LMIX_ATTN : (s == "lightning" ? LMIX_LIGHTNING : -1); }
+
+// config.json of a layer-list decoder: "architecture", "vocab", "width", "residual_mult", "norm".eps, "canon".taps and "layers":
+// [{"type", "mixer": {...}, "mlp": null | {"kind": "dense", "ff"} | {"kind": "moe", "expert": {"ff"}, "router": {"experts", "top"}}}]
+void Model::init_layered_config(const cmjson::Value& root) {
+    const std::string arch = root.string("architecture", "");
+    if (arch != "Korupel") throw CmError(CM_ERR_UNSUPPORTED, "architecture '" + arch + "' not implemented (Korupel)");
+    layered = true;
+    lay.reset(new Layered());
+    Layered& L = *lay;
+    cfg.model_type = "korupel";
+    cfg.V = (int)root.integer("vocab", 0);
+    cfg.H = (int)root.integer("width", 0);
+    if (const cmjson::Value* n = root.get("norm")) cfg.eps = (float)n->number("eps", 1e-6);
+    if (const cmjson::Value* c = root.get("canon")) L.taps = (int)c->integer("taps", 0);
+    L.mult = (float)root.number("residual_mult", 1.0);
+    const cmjson::Value* ls = root.get("layers");
+    if (!ls || ls->kind != cmjson::Value::Arr || ls->arr.empty()) throw CmError(CM_ERR_IO, "config.json: no layers");
+    if (cfg.V <= 0 || cfg.H <= 0) throw CmError(CM_ERR_IO, "config.json: vocab / width missing");
+    if (L.taps < 0 || L.taps > 64) throw CmError(CM_ERR_UNSUPPORTED, "canon.taps out of range");
+    for (auto& e : ls->arr) {
+        LayerSpec sp;
+        sp.mixer = act_of(e->string("type", ""));
+        if (sp.mixer < 0) throw CmError(CM_ERR_UNSUPPORTED, "layer type '" + e->string("type", "") + "' not implemented");
+        const cmjson::Value* mx = e->get("mixer");
+        if (!mx || mx->kind != cmjson::Value::Obj) throw CmError(CM_ERR_IO, "config.json: layer without mixer");
+        sp.heads = (int)mx->integer("heads", 0);
+        sp.kv_heads = (int)mx->integer("kv_heads", sp.heads);
+        sp.dim = (int)mx->integer("dim", 0);
+        sp.vdim = (int)mx->integer("vdim", sp.dim);
+        if (sp.heads <= 0 || sp.dim <= 0 || sp.vdim <= 0) throw CmError(CM_ERR_IO, "config.json: mixer sizes");
+        if (sp.mixer == LMIX_ATTN) {
+            if (sp.kv_heads <= 0 || sp.heads % sp.kv_heads) throw CmError(CM_ERR_INVALID, "heads % kv_heads != 0");
+            if (sp.vdim != sp.dim) throw CmError(CM_ERR_INVALID, "attention whose values are its keys needs vdim == dim");
+            if (sp.dim > 256) throw CmError(CM_ERR_UNSUPPORTED, "attention head size above 256");
+            sp.scale = (float)mx->number("scale", 1.0 / std::sqrt((double)sp.dim));
+            sp.win = 1ll << 40; sp.keep = 0;
+            if (const cmjson::Value* mk = mx->get("mask"))
+                if (mk->kind == cmjson::Value::Obj) {
+                    sp.win = mk->integer("size", sp.win);
+                    sp.keep = mk->integer("keep_first", 0);
+                }
+            if (sp.win <= 0 || sp.keep < 0) throw CmError(CM_ERR_INVALID, "mask.size / mask.keep_first");
+        } else {
+            if (sp.dim > 256) throw CmError(CM_ERR_UNSUPPORTED, "lightning head size above 256");
+            sp.kv_heads = sp.heads;
+            const cmjson::Value* dc = mx->get("decay");
+            if (dc && dc->kind == cmjson::Value::Arr) { for (auto& v : dc->arr) sp.decay.push_back((float)v->num); }
+            else sp.decay.assign((size_t)sp.heads, (float)mx->number("decay", 1.0));
+            if ((int)sp.decay.size() != sp.heads) throw CmError(CM_ERR_INVALID, "decay: one value per head");
+        }
+        const cmjson::Value* ml = e->get("mlp");
+        if (ml && ml->kind == cmjson::Value::Obj) {
+            const std::string kind = ml->string("kind", "dense");
+            if (kind == "dense") {
+                sp.mlp = LMLP_DENSE;
+                sp.ff = (int)ml->integer("ff", 0);
+            } else if (kind == "moe") {
+                sp.mlp = LMLP_MOE;
+                const cmjson::Value* ex = ml->get("expert");
+                const cmjson::Value* rt = ml->get("router");
+                if (!ex || !rt) throw CmError(CM_ERR_IO, "config.json: moe without expert / router");
+                sp.ff = (int)ex->integer("ff", 0);
+                sp.experts = (int)rt->integer("experts", 0);
+                sp.top = (int)rt->integer("top", 0);
+                if (sp.experts <= 0 || sp.top <= 0 || sp.top > sp.experts || sp.experts > 4096) throw CmError(CM_ERR_INVALID, "router.experts / router.top");
+            } else throw CmError(CM_ERR_UNSUPPORTED, "mlp.kind '" + kind + "' not implemented");
+            if (sp.ff <= 0) throw CmError(CM_ERR_IO, "config.json: ff");
+        }
+        L.spec.push_back(sp);
+    }
+    cfg.L = (int)L.spec.size();
+    // the family-wide fields of the other decoders do not exist here: neutral values for the shared set-up code
+    cfg.I = 8; cfg.Hq = 1; cfg.Hkv = 1; cfg.D = 128; cfg.rot_dim = 128; cfg.max_pos = 1 << 20; cfg.tie = false; cfg.qk_norm = false;
+    L.f32 = opts.compute_dtype == CM_COMPUTE_F32;
+    if (opts.compute_dtype > CM_COMPUTE_F32) throw CmError(CM_ERR_INVALID, "cm_opts.compute_dtype");
+    if (opts.tp_size > 1) throw CmError(CM_ERR_UNSUPPORTED, "tensor parallelism is not implemented for layer-list decoders");
+    if (opts.isq != 0) throw CmError(CM_ERR_UNSUPPORTED, "in-situ quantisation is not implemented for layer-list decoders");
+    // the key cache follows the number format: bfloat16 pages, or f32 pages in the float32 format
+    opts.kv_dtype = L.f32 ? CM_KV_F32 : CM_KV_BF16;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// weights
+// ---------------------------------------------------------------------------------------------------------------
+namespace {
+
+struct LaySource {
+    virtual ~LaySource() {}
+    // values of tensor `name` with exactly n elements (bf16-representable for matrices)
+    virtual std::vector<float> get(const std::string& name, size_t n, float synth_scale, float synth_off) = 0;
+};
+
+struct LayFileSource : LaySource {
+    cmst::Checkpoint ck;
+    explicit LayFileSource(const std::string& dir) : ck(dir) {}
+    std::vector<float> get(const std::string& name, size_t n, float, float) override {
+        const cmst::TensorView& t = ck.get(name);
+        if (t.numel() != (int64_t)n) throw CmError(CM_ERR_IO, "tensor " + name + ": unexpected shape");
+        std::vector<float> out(n);
+        if (t.dtype == "BF16") {
+            const uint16_t* p = (const uint16_t*)t.data;
+            for (size_t i = 0; i < n; ++i) { const uint32_t u = (uint32_t)p[i] << 16; memcpy(&out[i], &u, 4); }
+        } else if (t.dtype == "F32") {
+            memcpy(out.data(), t.data, n * 4);
+        } else throw CmError(CM_ERR_UNSUPPORTED, "tensor " + name + ": dtype " + t.dtype);
+        return out;
+    }
+};
+
+struct LaySynthSource : LaySource {
+    uint64_t seed;
+    explicit LaySynthSource(uint64_t s) : seed(s) {}
+    std::vector<float> get(const std::string& name, size_t n, float scale, float off) override {
+        uint64_t h = 1469598103934665603ull ^ seed;
+        for (char c : name) { h ^= (unsigned char)c; h *= 1099511628211ull; }
+        std::vector<float> out(n);
+        for (size_t i = 0; i < n; ++i) {
+            h ^= h << 13; h ^= h >> 7; h ^= h << 17;
+            // sum of four bytes: a bell-shaped value in [-2, 2) with unit-order spread
+            const int c = (int)((h & 0xFF) + ((h >> 8) & 0xFF) + ((h >> 16) & 0xFF) + ((h >> 24) & 0xFF)) - 510;
+            out[i] = off + scale * (float)c / 147.8f;
+        }
+        return out;
+    }
+};
+
+uint16_t to_bf16(float f) {
+    uint32_t u; memcpy(&u, &f, 4);
+    if ((u & 0x7F800000u) == 0x7F800000u) return (uint16_t)(u >> 16);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+}  // namespace
+
+static float* up_f32(Model& m, const std::vector<float>& v) {
+    float* d = m.dalloc<float>(v.size(), true);
+    CM_HIP(hipMemcpy(d, v.data(), v.size() * sizeof(float), hipMemcpyHostToDevice));
+    return d;
+}
+static uint16_t* up_bf16(Model& m, const std::vector<float>& v) {
+    std::vector<uint16_t> b(v.size());
+    for (size_t i = 0; i < v.size(); ++i) b[i] = to_bf16(v[i]);
+    uint16_t* d = m.dalloc<uint16_t>(b.size(), true);
+    CM_HIP(hipMemcpy(d, b.data(), b.size() * sizeof(uint16_t), hipMemcpyHostToDevice));
+    return d;
+}
+static void append(std::vector<float>& dst, const std::vector<float>& src) { dst.insert(dst.end(), src.begin(), src.end()); }
+
+static void build_layered(Model& m, LaySource& src) {
+    Layered& L = *m.lay;
+    const size_t W = (size_t)m.cfg.H, V = (size_t)m.cfg.V;
+    const float ws = 1.0f / std::sqrt((float)W);
+    m.embed = up_bf16(m, src.get("embed", V * W, 1.0f, 0.f));
+    L.w.resize(L.spec.size());
+    int kv_idx = 0;
+    for (size_t i = 0; i < L.spec.size(); ++i) {
+        const LayerSpec& sp = L.spec[i];
+        LayeredLayerW& w = L.w[i];
+        const std::string p = "l" + std::to_string(i) + ".";
+        w.norm1 = up_f32(m, src.get(p + "norm1", W, 0.1f, 1.f));
+        w.norm1b = up_f32(m, src.get(p + "norm1b", W, 0.1f, 1.f));
+        if (L.taps > 0) w.canon1 = up_f32(m, src.get(p + "canon1", W * L.taps, 0.3f, 0.f));
+        const size_t H = (size_t)sp.heads, G = (size_t)sp.kv_heads, d = (size_t)sp.dim, e = (size_t)sp.vdim;
+        std::vector<float> in, bias;
+        if (sp.mixer == LMIX_ATTN) {
+            w.q_off = 0; w.k_off = (int)(H * d); w.g_off = (int)(H * d + G * d); w.in_rows = (int)(H * d + G * d + H);
+            append(in, src.get(p + "mix.q", H * d * W, ws, 0.f));
+            append(in, src.get(p + "mix.k", G * d * W, ws, 0.f));
+            append(in, src.get(p + "mix.g", H * W, ws, 0.f));
+            append(bias, src.get(p + "mix.q.b", H * d, 0.1f, 0.f));
+            append(bias, src.get(p + "mix.k.b", G * d, 0.1f, 0.f));
+            bias.resize((size_t)w.in_rows, 0.f);
+            w.in_b = up_f32(m, bias);
+            w.r1 = up_f32(m, src.get(p + "mix.r1", H, 0.2f, 0.5f));
+            w.r2 = up_f32(m, src.get(p + "mix.r2", H, 0.1f, 0.5f));
+            w.o_w = up_bf16(m, src.get(p + "mix.o", W * H * d, 1.0f / std::sqrt((float)(H * d)), 0.f));
+            w.kv_idx = kv_idx++;
+        } else {
+            w.q_off = 0; w.k_off = (int)(H * d); w.v_off = (int)(2 * H * d); w.g_off = (int)(2 * H * d + H * e);
+            w.in_rows = (int)(2 * H * d + 2 * H * e);
+            append(in, src.get(p + "mix.q", H * d * W, ws, 0.f));
+            append(in, src.get(p + "mix.k", H * d * W, ws, 0.f));
+            append(in, src.get(p + "mix.v", H * e * W, ws, 0.f));
+            append(in, src.get(p + "mix.g", H * e * W, ws, 0.f));
+            w.mix_norm = up_f32(m, src.get(p + "mix.norm", H * e, 0.1f, 1.f));
+            w.o_w = up_bf16(m, src.get(p + "mix.o", W * H * e, 1.0f / std::sqrt((float)(H * e)), 0.f));
+            w.decay = up_f32(m, sp.decay);
+        }
+        w.in_w = up_bf16(m, in);
+        if (sp.mlp != LMLP_NONE) {
+            w.norm2 = up_f32(m, src.get(p + "norm2", W, 0.1f, 1.f));
+            w.norm2b = up_f32(m, src.get(p + "norm2b", W, 0.1f, 1.f));
+            if (L.taps > 0) w.canon2 = up_f32(m, src.get(p + "canon2", W * L.taps, 0.3f, 0.f));
+            const size_t ff = (size_t)sp.ff;
+            const float fs = 1.0f / std::sqrt((float)ff);
+            if (sp.mlp == LMLP_DENSE) {
+                w.gate = up_bf16(m, src.get(p + "mlp.gate", ff * W, ws, 0.f));
+                w.up = up_bf16(m, src.get(p + "mlp.up", ff * W, ws, 0.f));
+                w.down = up_bf16(m, src.get(p + "mlp.down", W * ff, fs, 0.f));
+            } else {
+                std::vector<float> g, u, dn;
+                for (int ex = 0; ex < sp.experts; ++ex) {
+                    const std::string q = p + "mlp.e" + std::to_string(ex) + ".";
+                    append(g, src.get(q + "gate", ff * W, ws, 0.f));
+                    append(u, src.get(q + "up", ff * W, ws, 0.f));
+                    append(dn, src.get(q + "down", W * ff, fs, 0.f));
+                }
+                w.gate = up_bf16(m, g); w.up = up_bf16(m, u); w.down = up_bf16(m, dn);
+                w.router = up_bf16(m, src.get(p + "mlp.router", (size_t)sp.experts * W, ws, 0.f));
+            }
+        }
+    }
+    L.final_norm = up_f32(m, src.get("final.norm", W, 0.1f, 1.f));
+    L.head = up_bf16(m, src.get("head", V * W, ws, 0.f));
+    m.lm_head = L.head;
+}
+
+void load_layered_from_dir(Model& m, const std::string& dir) {
+    try {
+        LayFileSource src(dir);
+        build_layered(m, src);
+    } catch (const CmError&) { throw; }
+    catch (const std::exception& e) { throw CmError(CM_ERR_IO, e.what()); }
+}
+void load_layered_synthetic(Model& m, uint64_t seed) {
+    LaySynthSource src(seed);
+    build_layered(m, src);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// runtime: key pages, state pools, scratch of one pass
+// ---------------------------------------------------------------------------------------------------------------
+void Model::alloc_runtime_layered() {
+    Layered& L = *lay;
+    const size_t W = (size_t)cfg.H;
+    kv_mode = L.f32 ? KV_F32 : KV_BF16;
+    kv_f32 = L.f32;
+    kv_esize = L.f32 ? 4 : 2;
+    // per-layer key pools (values are the keys: one pool per attention layer), page ids shared by all layers
+    size_t pool_bytes = 0, st = 0, cv = 0;
+    n_kv_layers = 0;
+    kv_index.assign((size_t)cfg.L, -1);
+    page_bytes = 0;
+    for (size_t i = 0; i < L.spec.size(); ++i) {
+        const LayerSpec& sp = L.spec[i];
+        LayeredLayerW& w = L.w[i];
+        if (sp.mixer == LMIX_ATTN) {
+            kv_index[i] = n_kv_layers++;
+            w.k_page_bytes = (size_t)sp.kv_heads * page * sp.dim * kv_esize;
+            w.k_pool_off = pool_bytes;
+            pool_bytes += (size_t)n_pages * w.k_page_bytes;
+            page_bytes += w.k_page_bytes;      // all layers' share of one page (kv_bytes)
+            const int nrep = sp.heads / sp.kv_heads;
+            if (std::find(L.nreps.begin(), L.nreps.end(), nrep) == L.nreps.end()) L.nreps.push_back(nrep);
+            L.max_o = std::max(L.max_o, sp.heads * sp.dim);
+        } else {
+            w.st_off = st;
+            st += (size_t)sp.heads * sp.dim * sp.vdim;
+            L.max_o = std::max(L.max_o, sp.heads * sp.vdim);
+        }
+        if (L.taps > 1) {
+            w.c1_off = cv; cv += (size_t)(L.taps - 1) * W;
+            if (sp.mlp != LMLP_NONE) { w.c2_off = cv; cv += (size_t)(L.taps - 1) * W; }
+        }
+        L.max_in = std::max(L.max_in, w.in_rows);
+        if (sp.mlp != LMLP_NONE) L.max_ff = std::max(L.max_ff, sp.ff);
+        if (sp.mlp == LMLP_MOE) { L.max_top = std::max(L.max_top, sp.top); L.max_E = std::max(L.max_E, sp.experts); }
+    }
+    kv_pool = (uint8_t*)dalloc<uint16_t>((pool_bytes + 1) / 2);
+    free_pages.resize((size_t)n_pages);
+    for (int64_t i = 0; i < n_pages; ++i) free_pages[(size_t)i] = (int32_t)(n_pages - 1 - i);
+    page_ref.assign((size_t)n_pages, 0);
+    conv_slot_elems = cv;
+    state_slot_elems = st;
+    if (cv) {
+        conv_pool = dalloc<float>(cv * seqs.size());
+        CM_HIP(hipMemsetAsync(conv_pool, 0, cv * seqs.size() * sizeof(float), stream));
+    }
+    if (st) {
+        state_pool = dalloc<float>(st * seqs.size());
+        CM_HIP(hipMemsetAsync(state_pool, 0, st * seqs.size() * sizeof(float), stream));
+    }
+    // scratch of one pass
+    L.cap = opts.prefill_chunk ? (int)opts.prefill_chunk : 2048;
+    L.cap = std::max(L.cap, 16);
+    chunk = L.cap;
+    const size_t cap = (size_t)L.cap;
+    L.X = dalloc<float>(cap * W);
+    L.Hn = dalloc<float>(cap * W);
+    L.Hc = dalloc<float>(cap * W);
+    L.Y = dalloc<float>(cap * W);
+    L.P = dalloc<float>(cap * (size_t)L.max_in);
+    L.O = dalloc<float>(cap * (size_t)L.max_o);
+    L.O2 = dalloc<float>(cap * (size_t)L.max_o);
+    if (L.max_ff) L.HH = dalloc<float>(cap * (size_t)L.max_top * (size_t)L.max_ff);
+    if (L.max_E > 1 || L.max_top > 1 || std::any_of(L.spec.begin(), L.spec.end(), [](const LayerSpec& s) { return s.mlp == LMLP_MOE; })) {
+        L.YS = dalloc<float>(cap * (size_t)L.max_top * W);
+        L.wsel = dalloc<float>(cap * (size_t)L.max_top);
+        L.sel = dalloc<int32_t>(cap * (size_t)L.max_top);
+        L.srt = dalloc<int32_t>(cap * (size_t)L.max_top);
+        L.off = dalloc<int32_t>((size_t)L.max_E + 1);
+    }
+    L.Xw = dalloc<float>((size_t)Layered::LOGIT_ROWS * W);
+    logitsb = dalloc<float>((size_t)Layered::LOGIT_ROWS * cfg.V);
+    logits = dalloc<float>((size_t)cfg.V);
+    V_l = cfg.V;
+    CM_HIP(hipHostMalloc((void**)&h_logits, (size_t)cfg.V * sizeof(float)));
+    CM_HIP(hipHostMalloc((void**)&L.h_rows, (size_t)Layered::LOGIT_ROWS * cfg.V * sizeof(float)));
+    L.d_greedy = dalloc<uint32_t>(Layered::LOGIT_ROWS);
+    CM_HIP(hipHostMalloc((void**)&L.h_greedy, Layered::LOGIT_ROWS * sizeof(uint32_t)));
+    // one table upload per pass: ids | rowseg | wanted rows | segments | page tables | attention tiles per group size
+    size_t tiles = 0;
+    for (int nrep : L.nreps) tiles += 2 * (cap * (size_t)nrep / 16 + (size_t)MAXB + 1);
+    L.tab_ints = 3 * cap + (size_t)MAXB * (sizeof(LaySegDev) / 4) + (size_t)MAXB * max_pages_per_seq + tiles + 64;
+    L.d_tab = dalloc<int32_t>(L.tab_ints);
+    CM_HIP(hipHostMalloc((void**)&L.h_tab, L.tab_ints * sizeof(int32_t)));
+    CM_HIP(hipStreamSynchronize(stream));
+}
+
+size_t Model::layered_capture(float* out, size_t n) const {
+    if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
+    const size_t k = std::min(n, lay->captured.size());
+    if (out && k) memcpy(out, lay->captured.data(), k * sizeof(float));
+    return lay->captured.size();
+}
+void Model::layered_set_capture(bool on) {
+    if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
+    lay->capture = on;
+    lay->captured.clear();
+}
+void Model::layered_cow_page(int32_t oldp, int32_t newp) {
+    Layered& L = *lay;
+    for (size_t i = 0; i < L.w.size(); ++i) {
+        const LayeredLayerW& w = L.w[i];
+        if (w.kv_idx < 0) continue;
+        CM_HIP(hipMemcpyAsync(kv_pool + w.k_pool_off + (size_t)newp * w.k_page_bytes, kv_pool + w.k_pool_off + (size_t)oldp * w.k_page_bytes,
+                              w.k_page_bytes, hipMemcpyDeviceToDevice, stream));
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// one step: every item appends its tokens to its sequence; all items run as one batch
+// ---------------------------------------------------------------------------------------------------------------
+namespace {
+struct PassSeg { size_t item; size_t off; int n; };
+}
+
+void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out, uint32_t* greedy_out) {
+    if (!layered) throw CmError(CM_ERR_UNSUPPORTED, "step_batch: not a layer-list decoder");
+    if (n_items == 0 || !items) throw CmError(CM_ERR_INVALID, "empty step");
+    Layered& L = *lay;
+    const int W = cfg.H, V = cfg.V;
+    hipStream_t s = stream;
+    for (size_t i = 0; i < n_items; ++i) {
+        const StepItem& it = items[i];
+        if (!it.ids || it.n == 0) throw CmError(CM_ERR_INVALID, "empty input");
+        Seq& q = seq(it.seq);
+        for (size_t c = 0; c < i; ++c) if (items[c].seq == it.seq) throw CmError(CM_ERR_INVALID, "sequence appears twice in one step");
+        if (q.len + (int64_t)it.n > (int64_t)max_seq) throw CmError(CM_ERR_RANGE, "sequence longer than max_seq_len");
+        for (size_t k = 0; k < it.n; ++k) if (it.ids[k] >= (uint32_t)V) throw CmError(CM_ERR_RANGE, "token id >= vocab_size");
+        for (int k = 0; k < it.n_want; ++k)
+            if (it.want[k] < 0 || (size_t)it.want[k] >= it.n || (k && it.want[k] <= it.want[k - 1]))
+                throw CmError(CM_ERR_INVALID, "wanted positions must ascend inside the portion");
+    }
+    // pages first: a step that does not fit changes nothing
+    {
+        size_t need = 0;
+        for (size_t i = 0; i < n_items; ++i) {
+            const Seq& q = seq(items[i].seq);
+            const size_t want = (size_t)((q.len + (int64_t)items[i].n + page - 1) / page);
+            if (want > q.pages.size()) need += want - q.pages.size();
+            if ((q.len % page) != 0 && !q.pages.empty() && page_ref[(size_t)q.pages[(size_t)(q.len / page)]] > 1) ++need;
+        }
+        if (need > free_pages.size()) throw CmError(CM_ERR_OOM, "KV pool exhausted");
+        for (size_t i = 0; i < n_items; ++i) ensure_pages(items[i].seq, seq(items[i].seq).len + (int64_t)items[i].n);
+    }
+    active_seq = -1; active_pages_uploaded = 0;
+    size_t out_row = 0;                       // next row of logits_out / greedy_out
+    size_t it_i = 0, it_off = 0;
+    while (it_i < n_items) {
+        // ---- cut the next pass: items in order, at most cap rows and MAXB segments
+        std::vector<PassSeg> ps;
+        int T = 0;
+        while (it_i < n_items && T < L.cap && (int)ps.size() < MAXB) {
+            const int n = (int)std::min<size_t>(items[it_i].n - it_off, (size_t)(L.cap - T));
+            ps.push_back(PassSeg{it_i, it_off, n});
+            T += n; it_off += (size_t)n;
+            if (it_off == items[it_i].n) { ++it_i; it_off = 0; }
+        }
+        const int nseg = (int)ps.size();
+        CM_HIP(hipStreamSynchronize(s));      // the pinned tables of the previous pass have been consumed
+        int32_t* tab = L.h_tab;
+        size_t o = 0;
+        int32_t* t_ids = tab + o; const size_t o_ids = o; o += (size_t)T;
+        int32_t* t_rowseg = tab + o; const size_t o_rowseg = o; o += (size_t)T;
+        int32_t* t_wrows = tab + o; const size_t o_wrows = o; o += (size_t)T;
+        LaySegDev* t_segs = (LaySegDev*)(tab + o); const size_t o_segs = o; o += (size_t)nseg * (sizeof(LaySegDev) / 4);
+        int32_t* t_bt = tab + o; const size_t o_bt = o; o += (size_t)nseg * max_pages_per_seq;
+        int nw = 0, row = 0;
+        bool all_decode = true;
+        for (int k = 0; k < nseg; ++k) {
+            const StepItem& it = items[ps[(size_t)k].item];
+            Seq& q = seq(it.seq);
+            const int n = ps[(size_t)k].n;
+            const int sp = (int)q.len;
+            t_segs[k] = LaySegDev{row, n, sp, it.seq, k * max_pages_per_seq, 0, 0, 0};
+            memcpy(t_bt + (size_t)k * max_pages_per_seq, q.pages.data(), q.pages.size() * sizeof(int32_t));
+            for (int r = 0; r < n; ++r) { t_ids[row + r] = (int32_t)it.ids[ps[(size_t)k].off + (size_t)r]; t_rowseg[row + r] = k; }
+            if (it.n_want < 0) { if (ps[(size_t)k].off + (size_t)n == it.n) t_wrows[nw++] = row + n - 1; }
+            else for (int j = 0; j < it.n_want; ++j) {
+                const long p = (long)it.want[j] - (long)ps[(size_t)k].off;
+                if (p >= 0 && p < n) t_wrows[nw++] = row + (int)p;
+            }
+            if (n != 1) all_decode = false;
+            row += n;
+            q.len += n;                        // the cache holds these positions once the pass has run
+        }
+        std::map<int, std::pair<size_t, int>> tiles;      // nrep -> (offset, count)
+        for (int nrep : L.nreps) {
+            if (o & 1) ++o;                    // int2 entries
+            const size_t o_t = o; int cnt = 0;
+            for (int k = 0; k < nseg; ++k)
+                for (int q0 = 0; q0 < t_segs[k].n * nrep; q0 += 16) { tab[o++] = k; tab[o++] = q0; ++cnt; }
+            tiles[nrep] = {o_t, cnt};
+        }
+        if (o > L.tab_ints) throw CmError(CM_ERR_INVALID, "step tables overflow");
+        CM_HIP(hipMemcpyAsync(L.d_tab, tab, o * sizeof(int32_t), hipMemcpyHostToDevice, s));
+        const uint32_t* d_ids = (const uint32_t*)(L.d_tab + o_ids);
+        const int32_t* d_rowseg = L.d_tab + o_rowseg;
+        const int32_t* d_wrows = L.d_tab + o_wrows;
+        const LaySegDev* d_segs = (const LaySegDev*)(L.d_tab + o_segs);
+        const int32_t* d_bt = L.d_tab + o_bt;
+
+        launch_embed_rows(embed, d_ids, L.X, T, W, V, s);
+        const bool bf = !L.f32;
+        auto norm_canon = [&](const float* nw_, const float* cw, size_t coff) {
+            if (L.taps <= 0) { launch_lay_rms_rows(L.X, nullptr, nw_, L.Hc, T, W, cfg.eps, s); return; }
+            if (all_decode) {
+                launch_lay_norm_canon_decode(L.X, nw_, cfg.eps, L.Hc, cw, conv_pool, conv_slot_elems, coff, d_segs, T, W, L.taps, s);
+                return;
+            }
+            launch_lay_rms_rows(L.X, nullptr, nw_, L.Hn, T, W, cfg.eps, s);
+            launch_lay_canon(L.Hn, L.Hc, cw, conv_pool, conv_slot_elems, coff, d_segs, d_rowseg, T, W, L.taps, s);
+            launch_lay_canon_tail(L.Hn, conv_pool, conv_slot_elems, coff, d_segs, nseg, W, L.taps, s);
+        };
+        for (size_t li = 0; li < L.spec.size(); ++li) {
+            const LayerSpec& sp = L.spec[li];
+            const LayeredLayerW& w = L.w[li];
+            norm_canon(w.norm1, w.canon1, w.c1_off);
+            LGemmArgs g;
+            g.A = L.Hc; g.lda = W; g.W = w.in_w; g.bias = w.in_b; g.C = L.P; g.ldc = w.in_rows; g.M = T; g.N = w.in_rows; g.K = W;
+            g.act_split = w.g_off; g.act2 = LACT_SIGMOID;
+            g.act = sp.mixer == LMIX_ATTN ? LACT_NONE : LACT_SILU;
+            launch_lgemm(g, bf, 1, s);
+            int on = 0;
+            const float* oa = nullptr;
+            if (sp.mixer == LMIX_ATTN) {
+                void* kp = kv_pool + w.k_pool_off;
+                launch_lay_k_append(L.P, w.in_rows, w.k_off, kp, kv_mode, d_bt, d_segs, d_rowseg, T, sp.kv_heads, sp.dim, page, s);
+                LAttnArgs a;
+                a.proj = L.P; a.ldp = w.in_rows; a.q_off = w.q_off; a.g_off = w.g_off;
+                a.out = L.O; a.ldo = sp.heads * sp.dim;
+                a.kpool = kp; a.bt = d_bt; a.segs = d_segs;
+                const auto& tl = tiles[sp.heads / sp.kv_heads];
+                a.tiles = (const int2*)(L.d_tab + tl.first); a.ntiles = tl.second;
+                a.r1 = w.r1; a.r2 = w.r2; a.H = sp.heads; a.G = sp.kv_heads; a.d = sp.dim; a.page = page;
+                a.scale = sp.scale; a.win = sp.win; a.keep = sp.keep;
+                launch_lay_attn(a, kv_mode, s);
+                on = sp.heads * sp.dim; oa = L.O;
+            } else {
+                LLightArgs a;
+                a.proj = L.P; a.ldp = w.in_rows; a.q_off = w.q_off; a.k_off = w.k_off; a.v_off = w.v_off;
+                a.out = L.O; a.ldo = sp.heads * sp.vdim;
+                a.state_pool = state_pool; a.slot_stride = state_slot_elems; a.st_off = w.st_off;
+                a.segs = d_segs; a.nseg = nseg; a.decay = w.decay; a.H = sp.heads; a.d = sp.dim; a.e = sp.vdim;
+                launch_lay_lightning(a, s);
+                on = sp.heads * sp.vdim;
+                launch_lay_rms_gate(L.O, L.P + w.g_off, w.in_rows, w.mix_norm, L.O2, T, on, cfg.eps, s);
+                oa = L.O2;
+            }
+            LGemmArgs go;
+            go.A = oa; go.lda = on; go.W = w.o_w; go.C = L.Y; go.ldc = W; go.M = T; go.N = W; go.K = on;
+            launch_lgemm(go, bf, 1, s);
+            launch_lay_post_norm(L.X, L.Y, w.norm1b, L.mult, cfg.eps, T, W, nullptr, 0, s);
+            if (sp.mlp != LMLP_NONE) {
+                norm_canon(w.norm2, w.canon2, w.c2_off);
+                if (sp.mlp == LMLP_DENSE) {
+                    LGemmArgs gu;
+                    gu.A = L.Hc; gu.lda = W; gu.W = w.gate; gu.W2 = w.up; gu.C = L.HH; gu.ldc = sp.ff; gu.M = T; gu.N = sp.ff; gu.K = W;
+                    gu.act = LACT_GELU_TANH;
+                    launch_lgemm(gu, bf, 1, s);
+                    LGemmArgs dn;
+                    dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.C = L.Y; dn.ldc = W; dn.M = T; dn.N = W; dn.K = sp.ff;
+                    launch_lgemm(dn, bf, 1, s);
+                    launch_lay_post_norm(L.X, L.Y, w.norm2b, L.mult, cfg.eps, T, W, nullptr, 0, s);
+                } else {
+                    launch_lay_router(L.Hc, w.router, L.sel, L.wsel, T, W, sp.experts, sp.top, s);
+                    launch_lay_moe_plan(L.sel, L.off, L.srt, T * sp.top, sp.experts, s);
+                    LGemmArgs gu;
+                    gu.A = L.Hc; gu.lda = W; gu.a_idx = L.srt; gu.a_div = sp.top;
+                    gu.W = w.gate; gu.W2 = w.up; gu.w_stride = (size_t)sp.ff * W;
+                    gu.C = L.HH; gu.ldc = sp.ff; gu.M = T; gu.N = sp.ff; gu.K = W; gu.grp_off = L.off; gu.act = LACT_SILU;
+                    launch_lgemm(gu, bf, sp.experts, s);
+                    LGemmArgs dn;
+                    dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.w_stride = (size_t)W * sp.ff;
+                    dn.C = L.YS; dn.ldc = W; dn.c_idx = L.srt; dn.M = T; dn.N = W; dn.K = sp.ff; dn.grp_off = L.off;
+                    launch_lgemm(dn, bf, sp.experts, s);
+                    launch_lay_post_norm(L.X, L.YS, w.norm2b, L.mult, cfg.eps, T, W, L.wsel, sp.top, s);
+                }
+            }
+            if (L.capture) {
+                const size_t at = L.captured.size();
+                L.captured.resize(at + (size_t)T * W);
+                CM_HIP(hipMemcpyAsync(L.captured.data() + at, L.X, (size_t)T * W * sizeof(float), hipMemcpyDeviceToHost, s));
+                CM_HIP(hipStreamSynchronize(s));
+            }
+        }
+        // ---- final norm + head over the wanted rows, LOGIT_ROWS at a time
+        for (int w0 = 0; w0 < nw; w0 += Layered::LOGIT_ROWS) {
+            const int nr = std::min(Layered::LOGIT_ROWS, nw - w0);
+            launch_lay_rms_rows(L.X, d_wrows + w0, L.final_norm, L.Xw, nr, W, cfg.eps, s);
+            LGemmArgs hd;
+            hd.A = L.Xw; hd.lda = W; hd.W = L.head; hd.C = logitsb; hd.ldc = V; hd.M = nr; hd.N = V; hd.K = W;
+            launch_lgemm(hd, bf, 1, s);
+            if (greedy_out) {
+                launch_lay_argmax_rows(logitsb, V, V, L.d_greedy, nr, s);
+                CM_HIP(hipMemcpyAsync(L.h_greedy, L.d_greedy, (size_t)nr * sizeof(uint32_t), hipMemcpyDeviceToHost, s));
+            }
+            if (logits_out) CM_HIP(hipMemcpyAsync(L.h_rows, logitsb, (size_t)nr * V * sizeof(float), hipMemcpyDeviceToHost, s));
+            if (greedy_out || logits_out || w0 + nr < nw) CM_HIP(hipStreamSynchronize(s));
+            if (greedy_out) memcpy(greedy_out + out_row, L.h_greedy, (size_t)nr * sizeof(uint32_t));
+            if (logits_out) memcpy(logits_out + out_row * (size_t)V, L.h_rows, (size_t)nr * V * sizeof(float));
+            out_row += (size_t)nr;
+        }
+    }
+    logits_gathered = true;
+    CM_HIP(hipStreamSynchronize(s));
+}
+
+// the entry points of the other families, for this one
+void Model::layered_forward(int sq, const uint32_t* ids, size_t n, size_t start_pos, float* logits_out, uint32_t* greedy_out) {
+    Seq& q = seq(sq);
+    if ((int64_t)start_pos > q.len) throw CmError(CM_ERR_RANGE, "start_pos beyond cached length");
+    if ((int64_t)start_pos < q.len) seq_truncate(sq, start_pos);     // only to 0: the recurrent state cannot be rewound
+    StepItem it{sq, ids, n, nullptr, -1};
+    uint32_t g = 0;
+    step_batch(&it, 1, logits_out, &g);
+    if (greedy_out) *greedy_out = g;
+    // the last row's logits are also what cm_sample / cm_read_logits look at
+    CM_HIP(hipMemcpyAsync(logits, logitsb, (size_t)cfg.V * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    CM_HIP(hipStreamSynchronize(stream));
+}
+
+uint64_t Model::layered_decode_bytes(size_t ctx) const {
+    const Layered& L = *lay;
+    const uint64_t W = (uint64_t)cfg.H;
+    uint64_t b = 2ull * (uint64_t)cfg.V * W + 2ull * W;       // head + one embedding row
+    for (size_t i = 0; i < L.spec.size(); ++i) {
+        const LayerSpec& sp = L.spec[i];
+        b += 2ull * (uint64_t)L.w[i].in_rows * W;
+        if (sp.mixer == LMIX_ATTN) {
+            b += 2ull * W * sp.heads * sp.dim;
+            const uint64_t seen = std::min<uint64_t>(ctx, (uint64_t)std::min<long long>(sp.win, 1ll << 40) + (uint64_t)sp.keep);
+            b += seen * (uint64_t)sp.kv_heads * sp.dim * kv_esize;
+        } else {
+            b += 2ull * W * sp.heads * sp.vdim + 8ull * sp.heads * sp.dim * sp.vdim;    // state read + write
+        }
+        if (sp.mlp == LMLP_DENSE) b += 6ull * W * sp.ff;
+        else if (sp.mlp == LMLP_MOE) b += 6ull * W * sp.ff * sp.top + 2ull * W * sp.experts;
+    }
+    return b;
+}
+
+}  // namespace cm

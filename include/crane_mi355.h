@@ -120,8 +120,13 @@ typedef struct cm_opts {
                                /*   kernels_tp.hip: no RCCL call in the token loop).  EXPERIMENTAL on distinct       */
                                /*   devices: never run on > 1 GPU; needs uncached / fine-grained device memory for   */
                                /*   the inboxes and fails with CM_ERR_UNSUPPORTED where the runtime has none.        */
-    uint32_t reserved[1];
+    uint32_t compute_dtype;    /* layer-list decoders (config "architecture" + "layers"): CM_COMPUTE_BF16 (0, default):      */
+                               /*   projections on the bf16 matrix cores with f32 accumulation, bf16 key pages;             */
+                               /*   CM_COMPUTE_F32: every product in true f32 (FMA), f32 key pages.  What such a model      */
+                               /*   defines as 32-bit (residual, norms, scores, recurrent state, router) is f32 in both.    */
 } cm_opts;
+
+enum { CM_COMPUTE_BF16 = 0u, CM_COMPUTE_F32 = 1u };
 
 enum { CM_TP_SPMD = 0u, CM_TP_IN_PROCESS = 1u };
 enum { CM_TP_COLL_DEFAULT = 0u, CM_TP_COLL_RCCL = 1u, CM_TP_COLL_PEER = 2u };
@@ -311,6 +316,23 @@ int cm_seq_forward(cm_model* m, int32_t seq, const uint32_t* ids, size_t n, size
  * the remaining combinations decode one sequence at a time. */
 int cm_decode_batch(cm_model* m, const int32_t* seqs, const uint32_t* last_tokens, size_t n,
                     float* logits_out, uint32_t* greedy_out);
+
+/* One step of a layer-list decoder (config "architecture" + "layers"): every item appends its next tokens to its sequence,
+ * continuing at the sequence's cached length, and ALL items run as one batch in one pass over the weights -- portions of
+ * prompts beside single decode tokens.  `want` lists the positions inside the portion (ascending) whose logits are asked
+ * for; n_want < 0 means the last one.  logits_out [wanted rows][vocab] and greedy_out [wanted rows] (arg-max, lowest index
+ * among equals) follow the order of the items and of their wanted positions; either may be NULL.  The logits at a position
+ * do not depend on how its sequence was cut into steps or on what else was in the batch, beyond rounding.  A step that
+ * does not fit in the page pool fails with CM_ERR_OOM and changes nothing. */
+typedef struct cm_step_item {
+    int32_t seq;
+    int32_t n_want;
+    const uint32_t* tokens;
+    size_t n_tokens;
+    const int32_t* want;
+} cm_step_item;
+int cm_step_batch(cm_model* m, const cm_step_item* items, size_t n, float* logits_out, uint32_t* greedy_out);
+
 
 /* Whole prompts of n sequences in ONE pass over the weights: sequence seqs[i] is cleared and prefilled with ids[i][0 .. lens[i])
  * from position 0 (what cm_seq_forward(seq, ids, n, 0, ...) does for one), together at most prefill_chunk tokens and 128
