@@ -139,6 +139,42 @@ CONFIGS.update({
 })
 
 
+# ---- layer-list decoders (config "architecture" + "layers"): Korupel -------------------------------------------------------
+def korupel_config(vocab: int, width: int, pattern: str, heads: int, kv_heads: int, dim: int, window: int, keep_first: int,
+                   lin_heads: int, lin_dim: int, lin_vdim: int, ff: int, experts: int = 0, top: int = 0, expert_ff: int = 0,
+                   taps: int = 4, residual_mult: float = 0.3, eps: float = 1e-6) -> dict:
+    """pattern: one letter per layer -- 'a' window attention, 'l' lightning attention; upper case: mixture of experts, lower
+    case: dense feed-forward.  Lightning head h of H decays with 1 - 2^-(1 + 8 h / (H - 1)): from fast to slow."""
+    layers = []
+    for ch in pattern:
+        if ch.lower() == "a":
+            mixer = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, mask=dict(size=window, keep_first=keep_first))
+            kind = "attention"
+        else:
+            decay = [round(1.0 - 0.5 ** (1 + 8 * h / max(1, lin_heads - 1)), 6) for h in range(lin_heads)]
+            mixer = dict(heads=lin_heads, dim=lin_dim, vdim=lin_vdim, decay=decay)
+            kind = "lightning"
+        mlp = (dict(kind="moe", expert=dict(ff=expert_ff), router=dict(experts=experts, top=top)) if ch.isupper()
+               else dict(kind="dense", ff=ff))
+        layers.append(dict(type=kind, mixer=mixer, mlp=mlp))
+    return dict(architecture="Korupel", vocab=vocab, width=width, residual_mult=residual_mult, norm=dict(eps=eps),
+                canon=dict(taps=taps), layers=layers)
+
+
+CONFIGS.update({
+    "tiny-korupel": korupel_config(320, 128, "aLlA", heads=4, kv_heads=2, dim=32, window=24, keep_first=3, lin_heads=2, lin_dim=16,
+                                   lin_vdim=32, ff=192, experts=4, top=2, expert_ff=48),
+    # widths of a 1 B-class hybrid (the Qwen3.5-0.8B text decoder's: 1024 wide, 3584 ff, 24 layers, 3 linear : 1 softmax), dense
+    "korupel-1b": korupel_config(32768, 1024, "llla" * 6, heads=8, kv_heads=2, dim=128, window=4096, keep_first=4, lin_heads=16,
+                                 lin_dim=128, lin_vdim=128, ff=3584),
+    # the same with 16 experts of 896, 4 per token (equal active width)
+    "korupel-1b-moe": korupel_config(32768, 1024, "LLLA" * 6, heads=8, kv_heads=2, dim=128, window=4096, keep_first=4, lin_heads=16,
+                                     lin_dim=128, lin_vdim=128, ff=3584, experts=16, top=4, expert_ff=896),
+    "korupel-1b-4l": korupel_config(32768, 1024, "llla", heads=8, kv_heads=2, dim=128, window=4096, keep_first=4, lin_heads=16,
+                                    lin_dim=128, lin_vdim=128, ff=3584),
+})
+
+
 def get_config(name: str) -> dict:
     if name not in CONFIGS:
         raise KeyError(f"unknown config {name!r}; have {sorted(CONFIGS)}")

@@ -35,6 +35,7 @@ struct Request {
     bool greedy_plain = false;          // temperature <= 0 and no penalties: the arg-max of the step itself
     int64_t eos[4] = {-1, -1, -1, -1};
     bool cancelled = false;
+    size_t fed = 0;                     // layer-list decoders: tokens of `tokens` the cache and the state hold (prompts are fed in portions)
 
     size_t num_generated() const { return tokens.size() - prompt_len; }
     bool last_is_eos() const {
@@ -53,6 +54,7 @@ struct Engine {
     long effective_max_running = -1;    // Scheduler::effective_max_running (None == -1)
     uint64_t next_id = 1;
     std::deque<uint64_t> waiting, running;
+    std::deque<uint64_t> prefilling;    // layer-list decoders: admitted, prompt not fully fed yet (they hold a slot and pages)
     std::unordered_map<uint64_t, Request> reqs;
     std::deque<cm_engine_event> events;
     cm_engine_stats stats{};
@@ -65,10 +67,12 @@ struct Engine {
     }
     void release(Request& r) {
         if (r.seq >= 0) { m->seq_free(r.seq); r.seq = -1; }
+        r.fed = 0;
     }
     void drop(uint64_t id) {
         waiting.erase(std::remove(waiting.begin(), waiting.end(), id), waiting.end());
         running.erase(std::remove(running.begin(), running.end(), id), running.end());
+        prefilling.erase(std::remove(prefilling.begin(), prefilling.end(), id), prefilling.end());
         reqs.erase(id);
     }
     void finish(uint64_t id, uint32_t reason) {                     // finish_sequence (engine/mod.rs:1265-1316)
@@ -293,11 +297,125 @@ struct Engine {
         }
     }
 
+    // Layer-list decoders: a step of the engine is ONE batch of the model's step function (Model::step_batch) -- the next token
+    // of every running sequence beside portions of the prompts being fed, oldest first, as many tokens as the pass has rows
+    // left (chunked prefill: a long prompt never stalls the running sequences, and several short prompts share a pass).  A
+    // request holds its slot and pages from its first portion on; only its last portion asks for logits.  Same queues, same
+    // eviction rule (longest running sequence, back of the queue, re-fed from its first token), same sampler rows.
+    void step_mixed() {
+        const size_t cap = effective_max_running >= 0 ? (size_t)effective_max_running : max_running;
+        size_t budget = (size_t)std::max(1, m->chunk), reserved = 0;
+        struct Part { uint64_t id; size_t n; bool last; bool decode; };
+        std::vector<Part> parts;
+        auto pages_needed = [&](const Request& r, size_t upto) {
+            const size_t have = r.seq >= 0 ? m->seq(r.seq).pages.size() : 0, want = pages_for(upto);
+            return want > have ? want - have : 0;
+        };
+        for (uint64_t id : std::vector<uint64_t>(running.begin(), running.end())) {
+            if (budget == 0 || parts.size() >= (size_t)Model::MAXB) break;
+            if (std::find(running.begin(), running.end(), id) == running.end()) continue;      // preempted by an earlier iteration
+            Request& r = req(id);
+            const size_t need = pages_needed(r, r.tokens.size());
+            if (need && !make_room(reserved + need, id)) { fail(id, CM_ERR_OOM, "KV pool exhausted"); continue; }
+            reserved += need;
+            parts.push_back({id, 1, true, true});
+            --budget;
+        }
+        auto feed = [&](uint64_t id) {
+            Request& r = req(id);
+            const size_t n = std::min(budget, r.tokens.size() - r.fed);
+            if (n == 0) return;
+            const size_t need = pages_needed(r, r.fed + n + (r.fed + n == r.tokens.size() ? 1 : 0));
+            if (need && !make_room(reserved + need, id)) {
+                // nobody left to evict: the prompt can never fit; otherwise it waits for a running sequence to finish
+                if (running.empty() && prefilling.size() <= 1) fail(id, CM_ERR_OOM, "prompt does not fit in the KV pool");
+                return;
+            }
+            reserved += need;
+            parts.push_back({id, n, r.fed + n == r.tokens.size(), false});
+            budget -= n;
+        };
+        for (uint64_t id : std::vector<uint64_t>(prefilling.begin(), prefilling.end())) {
+            if (budget == 0 || parts.size() >= (size_t)Model::MAXB) break;
+            feed(id);
+        }
+        while (budget > 0 && parts.size() < (size_t)Model::MAXB && !waiting.empty() && running.size() + prefilling.size() < cap) {
+            const uint64_t id = waiting.front();
+            Request& r = req(id);
+            try { r.seq = m->seq_alloc(); } catch (const CmError&) { break; }
+            r.fed = 0;
+            waiting.pop_front();
+            prefilling.push_back(id);
+            const size_t before = parts.size();
+            feed(id);
+            if (parts.size() == before) break;
+        }
+        // evictions above may have taken sequences that already had their part
+        parts.erase(std::remove_if(parts.begin(), parts.end(), [&](const Part& p) { return !reqs.count(p.id) || req(p.id).seq < 0; }), parts.end());
+        if (parts.empty()) return;
+        std::vector<Model::StepItem> items(parts.size());
+        size_t rows = 0;
+        for (size_t i = 0; i < parts.size(); ++i) {
+            Request& r = req(parts[i].id);
+            if (parts[i].decode) r.fed = r.tokens.size() - 1;
+            items[i] = Model::StepItem{r.seq, r.tokens.data() + r.fed, parts[i].n, nullptr, parts[i].last ? -1 : 0};
+            if (parts[i].last) ++rows;
+        }
+        std::vector<uint32_t> greedy(rows + 1), picked(rows + 1);
+        try {
+            m->step_batch(items.data(), items.size(), nullptr, greedy.data());
+            // the wanted rows of the pass sit in logitsb in the order of the items: one set of sampler launches, one host sync
+            std::vector<Model::SampleReq> srows;
+            size_t row = 0;
+            for (size_t i = 0; i < parts.size(); ++i) {
+                if (!parts[i].last) continue;
+                Request& r = req(parts[i].id);
+                if (!r.greedy_plain) {
+                    const size_t w = std::min(r.tokens.size(), (size_t)opts.repeat_last_n);
+                    cm_sample_params sp = r.sp;
+                    sp.repeat_last_n = 0;
+                    sp.draw = (uint32_t)r.num_generated();
+                    srows.push_back({(int)row, sp, r.tokens.data() + (r.tokens.size() - w), w, false, m->logitsb + row * (size_t)m->cfg.V});
+                }
+                ++row;
+            }
+            if (!srows.empty()) {
+                uint32_t got[Model::SAMPLE_SLOTS];
+                m->sample_enqueue_rows(srows.data(), (int)srows.size());
+                m->sample_collect((int)rows, got);
+                for (const auto& q : srows) picked[(size_t)q.slot] = got[q.slot];
+            }
+        } catch (const CmError& e) {
+            for (const Part& p : parts) if (reqs.count(p.id)) fail(p.id, e.code, e.what());
+            return;
+        }
+        size_t row = 0;
+        bool any_decode = false;
+        for (const Part& p : parts) {
+            Request& r = req(p.id);
+            r.fed += p.n;
+            if (p.decode) any_decode = true;
+            if (!p.last) continue;
+            const uint32_t t = r.greedy_plain ? greedy[row] : picked[row];
+            ++row;
+            r.tokens.push_back(t);
+            emit_token(r, t);
+            if (!p.decode) {
+                stats.prefill_steps++;
+                prefilling.erase(std::remove(prefilling.begin(), prefilling.end(), p.id), prefilling.end());
+                if (!r.should_stop()) running.push_back(p.id);
+            }
+            if (r.should_stop()) finish(p.id, r.last_is_eos() ? CM_FINISH_STOP : CM_FINISH_LENGTH);
+        }
+        if (any_decode) stats.decode_rounds++;
+    }
+
     void step() {
         // check_cancelled (engine/mod.rs:601-620)
         std::vector<uint64_t> gone;
         for (auto& kv : reqs) if (kv.second.cancelled) gone.push_back(kv.first);
         for (uint64_t id : gone) finish(id, CM_FINISH_CANCELLED);
+        if (m->layered) { step_mixed(); return; }
         // Scheduler::schedule (scheduler.rs:67-98)
         const size_t cap = effective_max_running >= 0 ? (size_t)effective_max_running : max_running;
         if (running.size() < cap && !waiting.empty()) {
@@ -447,7 +565,7 @@ int cm_engine_step_many(cm_engine* h, size_t max_steps, cm_engine_event* ev, siz
     // return n = 0 with work pending and the caller would spin forever
     // (the loop condition reads rank 0's queues only: every rank's engine is in the same state between steps)
     for (size_t i = 0; rc == CM_OK && i < max_steps && (e.events.size() + per_step <= cap || (i == 0 && e.events.empty())); ++i) {
-        if (e.waiting.empty() && e.running.empty()) break;
+        if (e.waiting.empty() && e.running.empty() && e.prefilling.empty()) break;
         rc = engine_all(h, [](cm::Engine& x) { x.step(); });
     }
     size_t k = 0;
@@ -458,7 +576,7 @@ int cm_engine_step_many(cm_engine* h, size_t max_steps, cm_engine_event* ev, siz
 
 int cm_engine_has_work(const cm_engine* h) {
     if (!h) return 0;
-    return (!h->e.waiting.empty() || !h->e.running.empty() || !h->e.events.empty()) ? 1 : 0;
+    return (!h->e.waiting.empty() || !h->e.running.empty() || !h->e.prefilling.empty() || !h->e.events.empty()) ? 1 : 0;
 }
 
 int cm_engine_get_stats(const cm_engine* h, cm_engine_stats* out) {

@@ -34,6 +34,18 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return t;
 }
 
+// embedding rows of any width (the shared gather moves four elements at a time)
+__global__ __launch_bounds__(256) void lay_embed_rows_kernel(const uint16_t* __restrict__ emb, const uint32_t* __restrict__ ids,
+                                                             float* __restrict__ x, int W, int V) {
+    uint32_t tok = ids[blockIdx.x];
+    if (tok >= (uint32_t)V) tok = 0;
+    for (int i = threadIdx.x; i < W; i += 256) x[(size_t)blockIdx.x * W + i] = bf16_to_f32(emb[(size_t)tok * W + i]);
+}
+void launch_lay_embed_rows(const uint16_t* emb, const uint32_t* ids, float* x, int T, int W, int V, hipStream_t s) {
+    if (T <= 0) return;
+    hipLaunchKernelGGL(lay_embed_rows_kernel, dim3((unsigned)T), dim3(256), 0, s, emb, ids, x, W, V);
+}
+
 // ------------------------------------------------------------------------------------------------------------------
 // row norms
 // ------------------------------------------------------------------------------------------------------------------

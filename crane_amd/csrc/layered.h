@@ -67,6 +67,7 @@ struct LGemmArgs {
 // bf16 = true: A rounded to bfloat16, matrix cores, f32 accumulation; false: f32 FMA throughout
 void launch_lgemm(const LGemmArgs& a, bool bf16, int groups, hipStream_t s);
 
+void launch_lay_embed_rows(const uint16_t* emb, const uint32_t* ids, float* x, int T, int W, int V, hipStream_t s);
 void launch_lay_rms_rows(const float* x, const int32_t* rows, const float* w, float* out, int n_rows, int W, float eps, hipStream_t s);
 // out = h + conv(h) over time per channel; the taps - 1 inputs before a portion come from the sequence's tail in conv_pool
 void launch_lay_canon(const float* h, float* out, const float* cw, const float* conv_pool, size_t slot_stride, size_t off,

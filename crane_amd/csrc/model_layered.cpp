@@ -482,7 +482,8 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
         const LaySegDev* d_segs = (const LaySegDev*)(L.d_tab + o_segs);
         const int32_t* d_bt = L.d_tab + o_bt;
 
-        launch_embed_rows(embed, d_ids, L.X, T, W, V, s);
+        if (W % 4 == 0) launch_embed_rows(embed, d_ids, L.X, T, W, V, s);
+        else launch_lay_embed_rows(embed, d_ids, L.X, T, W, V, s);
         const bool bf = !L.f32;
         auto norm_canon = [&](const float* nw_, const float* cw, size_t coff) {
             if (L.taps <= 0) { launch_lay_rms_rows(L.X, nullptr, nw_, L.Hc, T, W, cfg.eps, s); return; }

@@ -1,0 +1,354 @@
+"""GPU: the Korupel decoder in the library (kernels_layered.hip, model_layered.cpp, the engine's mixed steps) against the plain
+NumPy implementation oracle/korupel_oracle.py, on small configurations with random weights made here.
+
+float32 compute is the sharp comparison (TOL_F32 relative to the largest logit); bfloat16 compute is checked against the
+same oracle with the rounding's own allowance, and against itself across schedules."""
+import numpy as np
+import pytest
+
+from oracle import korupel_oracle as O
+from tests import korupel_util as U
+
+pytestmark = pytest.mark.gpu
+
+TOL_F32 = 2e-4
+TOL_BF16 = 6e-2
+
+
+def _load(tmp_path, cfg, P, dtype="float32", **kw):
+    from crane_amd.backend import Model
+    kw.setdefault("max_seq_len", 512)
+    kw.setdefault("max_seqs", 4)
+    return Model.from_pretrained(U.write_checkpoint(str(tmp_path / "ckpt"), cfg, P), compute_dtype=dtype, **kw)
+
+
+def _err(got, want):
+    want = np.asarray(want, np.float64)
+    return float(np.abs(np.asarray(got, np.float64) - want).max() / np.abs(want).max())
+
+
+def _all(n):
+    return list(range(n))
+
+
+SINGLE = {
+    "attention alone": U.config([U.layer("attention", None, **U.attn(heads=4, kv_heads=2, dim=16, size=9, keep_first=2))]),
+    "attention, one key head, no kept tokens": U.config([U.layer("attention", None, **U.attn(heads=3, kv_heads=1, dim=24, size=7, keep_first=0))], taps=1),
+    "lightning alone": U.config([U.layer("lightning", None, **U.light(heads=3, dim=8, vdim=24, decay=(0.3, 0.9, 0.999)))]),
+    "dense feed-forward": U.config([U.layer("lightning", U.DENSE, **U.light())], taps=2),
+    "experts": U.config([U.layer("attention", U.moe(experts=5, top=2, ff=24), **U.attn())], taps=5),
+    "every expert chosen": U.config([U.layer("lightning", U.moe(experts=3, top=3, ff=8), **U.light())]),
+    "one expert of many": U.config([U.layer("lightning", U.moe(experts=7, top=1, ff=16), **U.light())]),
+}
+
+
+@pytest.mark.parametrize("name", list(SINGLE))
+def test_each_mechanism_alone_whole_prompt_and_layer_rows(tmp_path, name):
+    cfg = SINGLE[name]
+    P = U.random_weights(cfg, 1)
+    toks = U.tokens(41, cfg["vocab"], 1)
+    want, layers = O.forward(cfg, P, toks, True)
+    m = _load(tmp_path, cfg, P)
+    try:
+        m.layer_capture(True)
+        s = m.seq_alloc()
+        got, greedy = m.step_batch([(s, toks, _all(len(toks)))])
+        rows = m.layer_rows().reshape(len(cfg["layers"]), len(toks), cfg["width"])
+        assert _err(rows, layers) < TOL_F32
+        assert _err(got, want) < TOL_F32
+        assert list(greedy) == [int(np.argmax(r)) for r in got]
+    finally:
+        m.close()
+
+
+def test_prefill_against_token_by_token_decoding(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 2)
+    toks = U.tokens(70, cfg["vocab"], 2)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        a, b = m.seq_alloc(), m.seq_alloc()
+        whole, _ = m.step_batch([(a, toks, _all(len(toks)))])
+        serial = np.concatenate([m.step_batch([(b, [t], [0])])[0] for t in toks])
+        assert _err(whole, want) < TOL_F32 and _err(serial, want) < TOL_F32
+        assert _err(serial, whole) < TOL_F32
+    finally:
+        m.close()
+
+
+@pytest.mark.parametrize("cuts", [[2] * 12 + [3, 5, 2, 7, 1, 1, 2, 16, 2], [64, 2, 1, 3], [1, 69], [33, 33, 4], [5, 60, 2, 2, 1]])
+def test_portions_of_several_sizes_down_to_two_tokens(tmp_path, cuts):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 3)
+    n = sum(cuts)
+    toks = U.tokens(n, cfg["vocab"], 3)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        s, at, out = m.seq_alloc(), 0, []
+        for c in cuts:
+            out.append(m.step_batch([(s, toks[at:at + c], _all(c))])[0])
+            at += c
+        assert m.seq_len(s) == n
+        assert _err(np.concatenate(out), want) < TOL_F32
+    finally:
+        m.close()
+
+
+def test_batches_of_unequal_requests_against_each_alone(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 4)
+    reqs = [U.tokens(n, cfg["vocab"], 10 + i) for i, n in enumerate((67, 5, 130, 31))]
+    want = [O.forward(cfg, P, t) for t in reqs]
+    # per step: (request, tokens taken) -- long portions beside single decode tokens, requests joining and pausing
+    plan = [[(0, 40), (1, 2)], [(0, 1), (1, 1), (2, 64)], [(2, 2), (0, 1), (3, 30)], [(1, 2), (2, 60), (3, 1), (0, 25)], [(2, 0)]]
+    m = _load(tmp_path, cfg, P)
+    try:
+        seqs = [m.seq_alloc() for _ in reqs]
+        at = [0] * len(reqs)
+        got = [[] for _ in reqs]
+        for step in plan:
+            step = [(r, c if c else len(reqs[r]) - at[r]) for r, c in step]
+            out, _ = m.step_batch([(seqs[r], reqs[r][at[r]:at[r] + c], _all(c)) for r, c in step])
+            row = 0
+            for r, c in step:
+                got[r].append(out[row:row + c])
+                row += c
+                at[r] += c
+        for r in range(len(reqs)):
+            have = np.concatenate(got[r])
+            assert _err(have, want[r][:len(have)]) < TOL_F32, r
+        assert at[2] == 130 and at[0] == 67
+    finally:
+        m.close()
+
+
+def test_pages_and_slots_that_are_freed_and_used_again(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 5)
+    m = _load(tmp_path, cfg, P, max_seq_len=192, kv_pool_tokens=256, max_seqs=2)        # 4 pages of 64, 2 slots
+    try:
+        for rnd in range(3):
+            reqs = [U.tokens(n, cfg["vocab"], 20 + 2 * rnd + i) for i, n in enumerate((100 + 7 * rnd, 90 - 11 * rnd))]
+            seqs = [m.seq_alloc(), m.seq_alloc()]
+            with pytest.raises(Exception):
+                m.seq_alloc()                                     # both slots taken
+            out, _ = m.step_batch([(seqs[0], reqs[0][:50], []), (seqs[1], reqs[1], _all(len(reqs[1])))])
+            assert _err(out, O.forward(cfg, P, reqs[1])) < TOL_F32
+            out, _ = m.step_batch([(seqs[0], reqs[0][50:], _all(len(reqs[0]) - 50))])
+            assert _err(out, O.forward(cfg, P, reqs[0])[50:]) < TOL_F32
+            assert m.active_kv_cache_bytes() > 0
+            for s in seqs:
+                m.seq_free(s)
+            assert m.active_kv_cache_bytes() == 0
+        # a step that does not fit in the pool fails and leaves the sequence as it was
+        a, b = m.seq_alloc(), m.seq_alloc()
+        m.step_batch([(a, U.tokens(150, cfg["vocab"], 1), None)])
+        with pytest.raises(Exception):
+            m.step_batch([(b, U.tokens(120, cfg["vocab"], 2), None)])
+        assert m.seq_len(b) == 0 and m.seq_len(a) == 150
+    finally:
+        m.close()
+
+
+def _planted(size, keep, heads=2, kv_heads=1, dim=16, alpha=9.0):
+    """One attention layer whose input is a function of the token alone (one tap, zero convolution), with a query token QT
+    and a key token KT whose score stands out by alpha^2 * scale whatever else is visible."""
+    cfg = U.config([U.layer("attention", None, **U.attn(heads=heads, kv_heads=kv_heads, dim=dim, size=size, keep_first=keep, scale=0.25))],
+                   vocab=67, width=40, taps=1)
+    P = U.random_weights(cfg, 7)
+    P["l0.canon1"][:] = 0
+    P["l0.mix.r1"][:] = U.bf16_round(np.full(heads, 0.05))
+    QT, KT = 65, 66
+    h = O.rms_norm(P["embed"].astype(np.float64), P["l0.norm1"], cfg["norm"]["eps"])
+    for g in range(kv_heads):
+        P["l0.mix.k"][g * dim] = U.bf16_round(alpha * h[KT] / (h[KT] @ h[KT]))
+    for hd in range(heads):
+        P["l0.mix.q"][hd * dim] = U.bf16_round(alpha * h[QT] / (h[QT] @ h[QT]))
+    return cfg, P, QT, KT
+
+
+@pytest.mark.parametrize("decoded", [False, True])
+def test_planted_keys_far_away_at_page_borders_and_at_both_edges_of_window_and_kept_tokens(tmp_path, decoded):
+    size, keep = 70, 3
+    cfg, P, QT, KT = _planted(size, keep)
+    m = _load(tmp_path, cfg, P)
+    try:
+        n = 200
+        # (key position, query position): kept token far back, first token that is not kept, window's oldest position and the
+        # one before it, keys on both sides of a page border (pages of 64 tokens)
+        cases = [(0, 199), (2, 150), (3, 150), (130, 199), (129, 199), (63, 64), (63, 132), (63, 133), (64, 133), (127, 128), (128, 197), (128, 198)]
+        for kp, qp in cases:
+            toks = U.tokens(n, 65, kp * 1000 + qp)
+            toks[kp], toks[qp] = KT, QT
+            want = O.forward(cfg, P, toks)
+            plain = list(toks)
+            plain[kp] = (toks[kp - 1] + 1) % 65 if kp else 1
+            moved = float(np.abs(O.forward(cfg, P, plain)[qp] - want[qp]).max() / np.abs(want[qp]).max())
+            seen = O.visible(qp, kp, size, keep)
+            assert (moved > 0.05) == seen, (kp, qp, moved)        # the planted key matters exactly when the mask shows it
+            s = m.seq_alloc()
+            if decoded:
+                m.step_batch([(s, toks[:qp - 2], [])])
+                got = np.concatenate([m.step_batch([(s, [toks[p]], [0])])[0] for p in range(qp - 2, qp + 1)])
+                assert _err(got, want[qp - 2:qp + 1]) < TOL_F32, (kp, qp)
+            else:
+                got, _ = m.step_batch([(s, toks[:qp + 1], [qp - 1, qp])])
+                assert _err(got, want[qp - 1:qp + 1]) < TOL_F32, (kp, qp)
+            m.seq_free(s)
+    finally:
+        m.close()
+
+
+def test_first_tokens_of_a_sequence(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 8)
+    m = _load(tmp_path, cfg, P)
+    try:
+        for n in (1, 2, 3, 5):
+            toks = U.tokens(n, cfg["vocab"], 40 + n)
+            s = m.seq_alloc()
+            got, _ = m.step_batch([(s, toks, _all(n))])
+            assert _err(got, O.forward(cfg, P, toks)) < TOL_F32
+            m.seq_free(s)
+        # a fresh slot starts from zero state although the one before it left its own behind
+        toks = U.tokens(4, cfg["vocab"], 50)
+        s = m.seq_alloc()
+        got = np.concatenate([m.step_batch([(s, [t], [0])])[0] for t in toks])
+        assert _err(got, O.forward(cfg, P, toks)) < TOL_F32
+    finally:
+        m.close()
+
+
+def test_long_decoding_past_the_window_many_times(tmp_path):
+    cfg = U.small_config()                                        # windows of 20 and 33 positions
+    P = U.random_weights(cfg, 9)
+    toks = U.tokens(230, cfg["vocab"], 9)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        s = m.seq_alloc()
+        m.step_batch([(s, toks[:10], [])])
+        got = np.concatenate([m.step_batch([(s, [t], [0])])[0] for t in toks[10:]])
+        assert _err(got, want[10:]) < TOL_F32
+    finally:
+        m.close()
+
+
+OTHER = {
+    "odd sizes": U.config([U.layer("attention", U.moe(experts=6, top=4, ff=10), **U.attn(heads=6, kv_heads=2, dim=12, size=1, keep_first=4, scale=1.0)),
+                           U.layer("lightning", None, **U.light(heads=1, dim=20, vdim=12, decay=(1.0,))),
+                           U.layer("attention", dict(kind="dense", ff=30), **U.attn(heads=1, kv_heads=1, dim=40, size=1000, keep_first=0))],
+                          vocab=37, width=30, taps=2, mult=1.0, eps=1e-5),
+    "wide heads": U.config([U.layer("lightning", U.DENSE, **U.light(heads=1, dim=160, vdim=72, decay=(0.97,))),
+                            U.layer("attention", None, **U.attn(heads=2, kv_heads=2, dim=192, size=16, keep_first=1))],
+                           vocab=50, width=64, taps=6, mult=0.5),
+    "lightning first, attention last": U.config([U.layer("lightning", U.moe(experts=2, top=1, ff=64), **U.light()),
+                                                 U.layer("lightning", U.DENSE, **U.light(heads=4, dim=4, vdim=4, decay=(0.1, 0.5, 0.9, 0.99))),
+                                                 U.layer("attention", U.DENSE, **U.attn(heads=8, kv_heads=8, dim=8, size=5, keep_first=5))],
+                                                vocab=128, width=64, taps=4),
+}
+
+
+@pytest.mark.parametrize("name", list(OTHER))
+def test_other_sizes_whole_portioned_and_decoded(tmp_path, name):
+    cfg = OTHER[name]
+    P = U.random_weights(cfg, 11)
+    toks = U.tokens(90, cfg["vocab"], 11)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        a, b = m.seq_alloc(), m.seq_alloc()
+        whole, _ = m.step_batch([(a, toks, _all(90))])
+        assert _err(whole, want) < TOL_F32
+        out, at = [], 0
+        for c in [7, 2, 30, 1, 1, 2, 40, 3, 1, 1, 1, 1]:
+            out.append(m.step_batch([(b, toks[at:at + c], _all(c))])[0])
+            at += c
+        assert at == 90 and _err(np.concatenate(out), want) < TOL_F32
+    finally:
+        m.close()
+
+
+def test_greedy_generation_through_generate_and_through_the_engine(tmp_path):
+    from crane_amd.backend import GenerationConfig
+    from crane_amd.engine import GenerationParams, InferenceEngine
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 12)
+    prompts = [U.tokens(n, cfg["vocab"], 60 + i) for i, n in enumerate((9, 70, 3, 25, 40))]
+    lens = [12, 6, 20, 9, 15]
+    want = [O.generate(cfg, P, p, n)[len(p):] for p, n in zip(prompts, lens)]
+    m = _load(tmp_path, cfg, P, max_seq_len=128, kv_pool_tokens=384, max_seqs=4, prefill_chunk=48)
+    try:
+        assert m.generate(prompts[0], GenerationConfig.greedy(lens[0]))[len(prompts[0]):] == want[0]
+        m.clear_kv_cache()
+        eng = InferenceEngine(m, max_running=3)                   # 5 requests, 3 slots, 48-row steps: prompts are fed in portions
+        ids = [eng.submit(p, GenerationParams.greedy(n)) for p, n in zip(prompts, lens)]
+        toks, done = eng.run_until_idle()
+        for rid, w in zip(ids, want):
+            assert toks[rid] == w
+            assert done[rid].kind == "finished" and done[rid].finish_reason == "length"
+        st = eng.stats()
+        assert st["completed"] == 5 and st["failed"] == 0 and st["free_pages"] == st["total_pages"]
+        # sampled requests run through the same steps and the device sampler
+        rid = eng.submit(prompts[3], GenerationParams(max_tokens=8, temperature=0.8, top_p=0.9, top_k=20, seed=5))
+        toks, done = eng.run_until_idle()
+        assert len(toks[rid]) == 8 and all(0 <= t < cfg["vocab"] for t in toks[rid])
+        eng.close()
+    finally:
+        m.close()
+
+
+def test_bfloat16_format_against_the_oracle_and_across_schedules(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 13)
+    toks = U.tokens(100, cfg["vocab"], 13)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P, dtype="bfloat16")
+    try:
+        a, b = m.seq_alloc(), m.seq_alloc()
+        whole, _ = m.step_batch([(a, toks, _all(100))])
+        assert _err(whole, want) < TOL_BF16
+        out, at = [], 0
+        for c in [50, 2, 13, 1, 1, 33]:
+            out.append(m.step_batch([(b, toks[at:at + c], _all(c))])[0])
+            at += c
+        assert _err(np.concatenate(out), want) < TOL_BF16
+        assert _err(np.concatenate(out), whole) < TOL_BF16
+    finally:
+        m.close()
+
+
+def test_fork_carries_pages_convolution_tails_and_linear_state(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 14)
+    toks = U.tokens(80, cfg["vocab"], 14)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        a = m.seq_alloc()
+        m.step_batch([(a, toks[:37], [])])
+        b = m.seq_fork(a)
+        ga, _ = m.step_batch([(a, toks[37:], _all(43)), ])
+        gb, _ = m.step_batch([(b, toks[37:], _all(43))])
+        assert _err(ga, want[37:]) < TOL_F32 and _err(gb, want[37:]) < TOL_F32
+        with pytest.raises(Exception):
+            m.seq_truncate(a, 10)                                 # a recurrent state cannot be rewound
+    finally:
+        m.close()
+
+
+def test_synthetic_registry_model_generates(tmp_path):
+    from crane_amd import configs
+    from crane_amd.backend import GenerationConfig, Model
+    m = Model.synthetic(configs.get_config("tiny-korupel"), seed=3, max_seq_len=128, max_seqs=2)
+    try:
+        assert m.num_layers() == 4 and m.vocab_size == 320
+        out = m.generate([1, 2, 3, 4, 5], GenerationConfig.greedy(6))
+        assert len(out) == 11
+        logits = m.forward_step([7, 8, 9], 0)[0, 0]
+        assert np.isfinite(logits).all() and int(np.argmax(logits)) == m.forward_step_greedy([7, 8, 9], 0)
+        assert m.decode_bytes_per_token(64) > m.weight_bytes() // 4
+    finally:
+        m.close()
