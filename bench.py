@@ -145,6 +145,75 @@ def relaunch_under_torchrun(n: int) -> int:
     return subprocess.call(cmd, env=env)
 
 
+def korupel_leg(args):
+    """--korupel: prompt and decode throughput of the Korupel decoder (layer-list family, crane_amd/csrc/model_layered.cpp) at the
+    widths of a real model, random weights, beside the closest family of the library at equal size: the Qwen3.5 hybrid (linear
+    attention 3 : 1 softmax attention, same width / ff / layers / vocabulary).  One JSON line; the default workload of this script
+    is not touched."""
+    import numpy as np
+    from crane_amd import configs
+    from crane_amd.backend import Model
+
+    def best(f, n=3):
+        ts = []
+        for _ in range(n):
+            t0 = time.perf_counter(); f(); ts.append(time.perf_counter() - t0)
+        return min(ts)
+
+    rows = []
+    ctx, K = args.ctx, args.steps
+    prompts = [int(x) for x in args.korupel_prompts.split(",")]
+    for name in args.korupel.split(","):
+        cfg = configs.get_config(name)
+        lay = cfg.get("architecture") == "Korupel"
+        V = cfg["vocab"] if lay else cfg["vocab_size"]
+        m = Model.synthetic(cfg, seed=0, max_seq_len=max(4096, ctx + K + 64), max_seqs=34, kv_dtype="bf16",
+                            prefill_split=1, **({"compute_dtype": "bfloat16"} if lay else {}))
+        r = {"model": name, "weight_bytes": m.weight_bytes(), "prefill": {}, "decode": {}}
+        ids = lambda n: [(7 * i + 3) % V for i in range(n)]
+        for n in prompts:
+            s = m.seq_alloc()
+            def run():
+                m.seq_truncate(s, 0)
+                m.seq_forward(s, ids(n), 0, want_logits=False)
+            run()
+            t = best(run)
+            m.seq_free(s)
+            # flops of the projections of n rows (the head runs on the last row only): 2 per bf16 weight outside the tables
+            w = (m.weight_bytes() - 2 * 2 * V * cfg["width" if lay else "hidden_size"]) / 2
+            r["prefill"][str(n)] = {"ms": round(t * 1e3, 3), "tok_s": round(n / t, 1), "mfma_frac": round(2 * w * n / t / (MFMA_PEAK_TFLOPS * 1e12), 4)}
+        # single-sequence greedy decode at ctx
+        m.clear_kv_cache()
+        m.forward_step(ids(ctx), 0)
+        m.bench_decode(5, min(16, K))
+        toks, ms = m.bench_decode(5, K)
+        bts = m.decode_bytes_per_token(ctx + K // 2)
+        r["decode"]["1"] = {"ctx": ctx, "ms_per_token": round(ms / K, 4), "tok_s": round(K / (ms / 1e3), 1),
+                            "hbm_frac": round(bts / (ms / K / 1e3) / (HBM_PEAK_GBS * 1e9), 4)}
+        # 32 sequences, one token each per step
+        m.clear_kv_cache()
+        B = 32
+        seqs = [m.seq_alloc() for _ in range(B)]
+        m.prefill_batch(seqs, [ids(48 + i) for i in range(B)], want_logits=False)
+        tk = [5] * B
+        def round_():
+            nonlocal tk
+            _, g = m.step_batch_decode(seqs, tk, want_logits=False)
+            tk = [int(x) for x in g]
+        for _ in range(3):
+            round_()
+        t0 = time.perf_counter()
+        for _ in range(max(8, K // 4)):
+            round_()
+        dt = (time.perf_counter() - t0) / max(8, K // 4)
+        r["decode"]["32"] = {"ms_per_round": round(dt * 1e3, 3), "tok_s": round(B / dt, 1)}
+        m.close()
+        rows.append(r)
+    print(json.dumps({"metric": "korupel prompt / decode throughput beside the closest family at equal size", "unit": "tokens/s",
+                      "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -175,7 +244,12 @@ def main():
     ap.add_argument("--force-rccl", action="store_true", help="TP=1 with every reduction routed through a 1-rank RCCL communicator "
                     "(CM_DEBUG_FORCE_RCCL): per-call enqueue cost of the collectives, one GPU")
     ap.add_argument("--isq", default=None, help="in-situ weight quantisation (q8_0): a DIFFERENT workload than the bf16 headline")
+    ap.add_argument("--korupel", default=None, metavar="CONFIGS", help="comma-separated registry configs (e.g. korupel-1b,qwen3.5-0.8b): "
+                    "prompt and decode throughput of each instead of the headline workload")
+    ap.add_argument("--korupel-prompts", default="512,2048", help="prompt lengths of --korupel")
     args = ap.parse_args()
+    if args.korupel:
+        sys.exit(korupel_leg(args))
 
     if args.tp_inprocess:      # ranks that share a device need one hardware queue per rank stream: before the HIP runtime starts
         os.environ.setdefault("GPU_MAX_HW_QUEUES", "16")

@@ -164,11 +164,11 @@ def korupel_config(vocab: int, width: int, pattern: str, heads: int, kv_heads: i
 CONFIGS.update({
     "tiny-korupel": korupel_config(320, 128, "aLlA", heads=4, kv_heads=2, dim=32, window=24, keep_first=3, lin_heads=2, lin_dim=16,
                                    lin_vdim=32, ff=192, experts=4, top=2, expert_ff=48),
-    # widths of a 1 B-class hybrid (the Qwen3.5-0.8B text decoder's: 1024 wide, 3584 ff, 24 layers, 3 linear : 1 softmax), dense
-    "korupel-1b": korupel_config(32768, 1024, "llla" * 6, heads=8, kv_heads=2, dim=128, window=4096, keep_first=4, lin_heads=16,
+    # the widths of the Qwen3.5-0.8B text decoder (1024 wide, 3584 ff, 24 layers, 3 linear : 1 softmax, vocabulary 248 320), dense
+    "korupel-1b": korupel_config(248320, 1024, "llla" * 6, heads=8, kv_heads=2, dim=128, window=4096, keep_first=4, lin_heads=16,
                                  lin_dim=128, lin_vdim=128, ff=3584),
     # the same with 16 experts of 896, 4 per token (equal active width)
-    "korupel-1b-moe": korupel_config(32768, 1024, "LLLA" * 6, heads=8, kv_heads=2, dim=128, window=4096, keep_first=4, lin_heads=16,
+    "korupel-1b-moe": korupel_config(248320, 1024, "LLLA" * 6, heads=8, kv_heads=2, dim=128, window=4096, keep_first=4, lin_heads=16,
                                      lin_dim=128, lin_vdim=128, ff=3584, experts=16, top=4, expert_ff=896),
     "korupel-1b-4l": korupel_config(32768, 1024, "llla", heads=8, kv_heads=2, dim=128, window=4096, keep_first=4, lin_heads=16,
                                     lin_dim=128, lin_vdim=128, ff=3584),

@@ -360,8 +360,135 @@ __global__ __launch_bounds__(256) void lgemm_bf16_kernel(LGemmArgs a) {
     }
 }
 
+// few rows (decode steps): the matrix is streamed ONCE with 16-byte non-temporal loads, one wave per two output columns, every
+// row of A (at most LV_MAXM, L2-resident) against each weight fragment; the wave's lanes split K.  bfloat16 format: A is rounded
+// on the fly, so a row gives the same products here and in the tiled kernel.
+constexpr int LV_MAXM = 8;
+template <bool BF16, bool DUAL>
+__global__ __launch_bounds__(256) void lgemv_kernel(LGemmArgs a) {
+    const int g = blockIdx.z;
+    int base = 0, rows = a.M;
+    if (a.grp_off) { base = a.grp_off[g]; rows = a.grp_off[g + 1] - base; }
+    if (rows <= 0) return;
+    rows = min(rows, LV_MAXM);
+    const uint16_t* W = a.W + (size_t)g * a.w_stride;
+    const uint16_t* W2 = DUAL ? a.W2 + (size_t)g * a.w_stride : nullptr;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = (blockIdx.x * 4 + wave) * 2;
+    if (n0 >= a.N) return;
+    const int n1 = min(n0 + 1, a.N - 1);                 // odd N: the second column repeats the first and is not stored
+    size_t ar[LV_MAXM];
+#pragma unroll
+    for (int r = 0; r < LV_MAXM; ++r) {
+        const int p = base + min(r, rows - 1);
+        ar[r] = (size_t)(a.a_idx ? a.a_idx[p] / a.a_div : p) * a.lda;
+    }
+    float acc[2][LV_MAXM] = {}, acc2[2][LV_MAXM] = {};
+    const int K = a.K;
+    const bool vec = (K % 8) == 0 && (a.lda % 4) == 0 && ((uintptr_t)a.A % 16) == 0 && ((uintptr_t)W % 16) == 0 &&
+                     (!DUAL || ((uintptr_t)W2 % 16) == 0);
+    if (vec) {
+        for (int k = lane * 8; k < K; k += 512) {
+            const u32x4 w0 = ld_nt16(W + (size_t)n0 * K + k), w1 = ld_nt16(W + (size_t)n1 * K + k);
+            u32x4 v0 = {0u, 0u, 0u, 0u}, v1 = {0u, 0u, 0u, 0u};
+            if (DUAL) { v0 = ld_nt16(W2 + (size_t)n0 * K + k); v1 = ld_nt16(W2 + (size_t)n1 * K + k); }
+#pragma unroll
+            for (int r = 0; r < LV_MAXM; ++r) {
+                if (r < rows) {
+                    const float4 xa = *(const float4*)(a.A + ar[r] + k), xb = *(const float4*)(a.A + ar[r] + k + 4);
+                    float x[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+                    if (BF16) {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) x[i] = bf16_round(x[i]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        acc[0][r] = fmaf(bf16_lo(w0[i]), x[2 * i], acc[0][r]); acc[0][r] = fmaf(bf16_hi(w0[i]), x[2 * i + 1], acc[0][r]);
+                        acc[1][r] = fmaf(bf16_lo(w1[i]), x[2 * i], acc[1][r]); acc[1][r] = fmaf(bf16_hi(w1[i]), x[2 * i + 1], acc[1][r]);
+                        if (DUAL) {
+                            acc2[0][r] = fmaf(bf16_lo(v0[i]), x[2 * i], acc2[0][r]); acc2[0][r] = fmaf(bf16_hi(v0[i]), x[2 * i + 1], acc2[0][r]);
+                            acc2[1][r] = fmaf(bf16_lo(v1[i]), x[2 * i], acc2[1][r]); acc2[1][r] = fmaf(bf16_hi(v1[i]), x[2 * i + 1], acc2[1][r]);
+                        }
+                    }
+                }
+            }
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) {
+            const float w0 = bf16_to_f32(W[(size_t)n0 * K + k]), w1 = bf16_to_f32(W[(size_t)n1 * K + k]);
+            const float v0 = DUAL ? bf16_to_f32(W2[(size_t)n0 * K + k]) : 0.f, v1 = DUAL ? bf16_to_f32(W2[(size_t)n1 * K + k]) : 0.f;
+#pragma unroll
+            for (int r = 0; r < LV_MAXM; ++r) {
+                if (r < rows) {
+                    float x = a.A[ar[r] + k];
+                    if (BF16) x = bf16_round(x);
+                    acc[0][r] = fmaf(w0, x, acc[0][r]); acc[1][r] = fmaf(w1, x, acc[1][r]);
+                    if (DUAL) { acc2[0][r] = fmaf(v0, x, acc2[0][r]); acc2[1][r] = fmaf(v1, x, acc2[1][r]); }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < LV_MAXM; ++r) {
+        if (r < rows) {
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const float v = wave_sum(acc[c][r]);
+                const float v2 = DUAL ? wave_sum(acc2[c][r]) : 0.f;
+                if (lane == 0 && (c == 0 || n0 + 1 < a.N)) lg_store(a, base + r, n0 + c, v, v2, DUAL);
+            }
+        }
+    }
+}
+
+// the column-range activation of a finished product, in place (products that ran on the shared GEMM kernels)
+__global__ __launch_bounds__(256) void lay_act_cols_kernel(float* __restrict__ C, int ldc, int N, int act, int act2, int split) {
+    const int n = blockIdx.y * 256 + threadIdx.x;
+    if (n >= N) return;
+    float* p = C + (size_t)blockIdx.x * ldc + n;
+    *p = lay_act(*p, n < split ? act : act2);
+}
+void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int split, hipStream_t s) {
+    if (M <= 0 || (act == LACT_NONE && (act2 == LACT_NONE || split >= N))) return;
+    hipLaunchKernelGGL(lay_act_cols_kernel, dim3((unsigned)M, (unsigned)((N + 255) / 256)), dim3(256), 0, s, C, ldc, N, act, act2, split);
+}
+// out = act(g) * u
+__global__ __launch_bounds__(256) void lay_act_mul_kernel(const float* __restrict__ g, const float* __restrict__ u, float* __restrict__ out,
+                                                          size_t n, int act) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = lay_act(g[i], act) * u[i];
+}
+void launch_lay_act_mul(const float* g, const float* u, float* out, size_t n, int act, hipStream_t s) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(lay_act_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, g, u, out, n, act);
+}
+// rows of f32 -> bfloat16 (round to nearest even): the A operand of the shared matrix-core GEMM
+__global__ __launch_bounds__(256) void lay_round_rows_kernel(const float* __restrict__ x, int ldx, uint16_t* __restrict__ out, int K) {
+    const float* xr = x + (size_t)blockIdx.x * ldx;
+    for (int k = threadIdx.x * 2; k < K; k += 512) {
+        const uint32_t pk = pack_bf16x2(xr[k], k + 1 < K ? xr[k + 1] : 0.f);
+        if (k + 1 < K) *(uint32_t*)(out + (size_t)blockIdx.x * K + k) = pk;
+        else out[(size_t)blockIdx.x * K + k] = (uint16_t)(pk & 0xFFFFu);
+    }
+}
+void launch_lay_round_rows(const float* x, int ldx, uint16_t* out, int M, int K, hipStream_t s) {
+    if (M <= 0) return;
+    hipLaunchKernelGGL(lay_round_rows_kernel, dim3((unsigned)M), dim3(256), 0, s, x, ldx, out, K);
+}
+
 void launch_lgemm(const LGemmArgs& a, bool bf16, int groups, hipStream_t s) {
     if (a.M <= 0 || a.N <= 0 || groups <= 0) return;
+    if (a.M <= LV_MAXM) {
+        const dim3 gv((unsigned)((a.N + 7) / 8), 1, (unsigned)groups);
+        if (bf16) {
+            if (a.W2) hipLaunchKernelGGL((lgemv_kernel<true, true>), gv, dim3(256), 0, s, a);
+            else hipLaunchKernelGGL((lgemv_kernel<true, false>), gv, dim3(256), 0, s, a);
+        } else {
+            if (a.W2) hipLaunchKernelGGL((lgemv_kernel<false, true>), gv, dim3(256), 0, s, a);
+            else hipLaunchKernelGGL((lgemv_kernel<false, false>), gv, dim3(256), 0, s, a);
+        }
+        return;
+    }
     const dim3 grid((unsigned)((a.M + LG_BM - 1) / LG_BM), (unsigned)((a.N + LG_BN - 1) / LG_BN), (unsigned)groups);
     if (bf16) {
         if (a.W2) hipLaunchKernelGGL(lgemm_bf16_kernel<true>, grid, dim3(256), 0, s, a);

@@ -64,9 +64,13 @@ struct LGemmArgs {
     const int32_t* grp_off = nullptr;                // grouped: rows [grp_off[g], grp_off[g + 1]) use matrix g; M bounds a group's rows
     int act = LACT_NONE, act2 = LACT_NONE, act_split = 0;   // columns < act_split: act, the others act2 (W2: act on the first product)
 };
-// bf16 = true: A rounded to bfloat16, matrix cores, f32 accumulation; false: f32 FMA throughout
+// bf16 = true: A rounded to bfloat16, matrix cores, f32 accumulation; false: f32 FMA throughout.  Up to 8 rows (per group): the
+// streaming row kernel instead of tiles.
 void launch_lgemm(const LGemmArgs& a, bool bf16, int groups, hipStream_t s);
 
+void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int split, hipStream_t s);
+void launch_lay_act_mul(const float* g, const float* u, float* out, size_t n, int act, hipStream_t s);
+void launch_lay_round_rows(const float* x, int ldx, uint16_t* out, int M, int K, hipStream_t s);
 void launch_lay_embed_rows(const uint16_t* emb, const uint32_t* ids, float* x, int T, int W, int V, hipStream_t s);
 void launch_lay_rms_rows(const float* x, const int32_t* rows, const float* w, float* out, int n_rows, int W, float eps, hipStream_t s);
 // out = h + conv(h) over time per channel; the taps - 1 inputs before a portion come from the sequence's tail in conv_pool

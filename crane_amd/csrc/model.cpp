@@ -775,8 +775,11 @@ void Model::cow_page(int s, size_t idx) {
     q.pages[idx] = newp;
     if (layered) { layered_cow_page(oldp, newp); if (active_seq == s) active_pages_uploaded = std::min(active_pages_uploaded, idx); return; }
     const size_t pitch = (size_t)n_pages * page_bytes;
-    CM_HIP(hipMemcpy2DAsync(kv_pool + (size_t)newp * page_bytes, pitch, kv_pool + (size_t)oldp * page_bytes, pitch,
-                            page_bytes, (size_t)n_kv_layers * 2, hipMemcpyDeviceToDevice, stream));
+    // one plain copy per (layer, K | V) plane of the pool (a pitched 2-D copy of the same bytes was the first call of two test
+    // runs that ended with a device error on the GPU boxes; plain device-to-device copies are what the other paths use)
+    for (size_t pl = 0; pl < (size_t)n_kv_layers * 2; ++pl)
+        CM_HIP(hipMemcpyAsync(kv_pool + pl * pitch + (size_t)newp * page_bytes, kv_pool + pl * pitch + (size_t)oldp * page_bytes,
+                              page_bytes, hipMemcpyDeviceToDevice, stream));
     if (active_seq == s) active_pages_uploaded = std::min(active_pages_uploaded, idx);    // re-upload the table entry
 }
 

@@ -36,6 +36,11 @@ struct Layered {
     int32_t *d_tab = nullptr, *h_tab = nullptr;
     size_t tab_ints = 0;
     static constexpr int LOGIT_ROWS = 256;
+    // bfloat16 format, products of 32 rows or more whose shape fits (N % 128 == 0, K % 32 == 0): the matrix-core GEMM the other
+    // families' prompt passes use (kernels_prefill.hip / kernels_gemm256.hip), plain bf16 activations; cm_debug_set("lay_shared_gemm", 0): never
+    bool shared_gemm = true;
+    uint16_t* Abf = nullptr;           // [cap rounded up to 256][widest K] bf16 A operand
+    float *G1 = nullptr, *G2 = nullptr;   // [cap][widest dense ff] the two products of a gated feed-forward
     bool capture = false;              // cm_debug_set("lay_capture"): keep the residual stream after every layer of every pass
     std::vector<float> captured;
     ~Layered() {
@@ -46,6 +51,27 @@ struct Layered {
 };
 
 void LayeredDeleter::operator()(Layered* p) const { delete p; }
+
+// one projection of a pass: the shared matrix-core GEMM where it applies, else the kernels of kernels_layered.hip
+static void lay_gemm(Model& m, Layered& L, const LGemmArgs& g, int groups, hipStream_t s) {
+    const bool bf = !L.f32;
+    if (bf && L.shared_gemm && L.Abf && groups == 1 && !g.a_idx && !g.c_idx && !g.grp_off && g.M >= 32 && g.N % 128 == 0 && g.K % 32 == 0 &&
+        (!g.W2 || (g.ldc == g.N && L.G1 && L.G2))) {
+        launch_lay_round_rows(g.A, g.lda, L.Abf, g.M, g.K, s);
+        GemmArgs a{};
+        a.A_hi = L.Abf; a.A_lo = nullptr; a.W = g.W; a.bias = g.bias;
+        a.C = g.W2 ? L.G1 : g.C; a.ldc = g.W2 ? g.N : g.ldc;
+        a.M = g.M; a.N = g.N; a.K = g.K; a.ws = m.pWS; a.ws_floats = m.pWS ? Model::gemm_ws_floats : 0; a.ksplit = 1; a.wide256 = m.gemm256;
+        bool ok = launch_gemm(a, GEPI_STORE, s);
+        if (ok && g.W2) { a.W = g.W2; a.C = L.G2; ok = launch_gemm(a, GEPI_STORE, s); }
+        if (ok) {
+            if (g.W2) launch_lay_act_mul(L.G1, L.G2, g.C, (size_t)g.M * g.N, g.act, s);
+            else launch_lay_act_cols(g.C, g.ldc, g.M, g.N, g.act, g.act2, g.act_split, s);
+            return;
+        }
+    }
+    launch_lgemm(g, bf, groups, s);
+}
 
 static int act_of(const std::string& s) { return s == "attention" ? LMIX_ATTN : (s == "lightning" ? LMIX_LIGHTNING : -1); }
 
@@ -351,6 +377,15 @@ void Model::alloc_runtime_layered() {
         L.srt = dalloc<int32_t>(cap * (size_t)L.max_top);
         L.off = dalloc<int32_t>((size_t)L.max_E + 1);
     }
+    if (!L.f32) {
+        int max_k = std::max((int)W, std::max(L.max_o, L.max_ff)), dense_ff = 0;
+        for (const LayerSpec& sp : L.spec) if (sp.mlp == LMLP_DENSE) dense_ff = std::max(dense_ff, sp.ff);
+        const size_t rows = (cap + 255) / 256 * 256;
+        L.Abf = dalloc<uint16_t>(rows * (size_t)max_k);
+        CM_HIP(hipMemsetAsync(L.Abf, 0, rows * (size_t)max_k * sizeof(uint16_t), stream));
+        if (dense_ff) { L.G1 = dalloc<float>(cap * (size_t)dense_ff); L.G2 = dalloc<float>(cap * (size_t)dense_ff); }
+        ensure_gemm_workspace();
+    }
     L.Xw = dalloc<float>((size_t)Layered::LOGIT_ROWS * W);
     logitsb = dalloc<float>((size_t)Layered::LOGIT_ROWS * cfg.V);
     logits = dalloc<float>((size_t)cfg.V);
@@ -373,6 +408,10 @@ size_t Model::layered_capture(float* out, size_t n) const {
     const size_t k = std::min(n, lay->captured.size());
     if (out && k) memcpy(out, lay->captured.data(), k * sizeof(float));
     return lay->captured.size();
+}
+void Model::layered_set_shared_gemm(bool on) {
+    if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
+    lay->shared_gemm = on;
 }
 void Model::layered_set_capture(bool on) {
     if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
@@ -484,7 +523,6 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
 
         if (W % 4 == 0) launch_embed_rows(embed, d_ids, L.X, T, W, V, s);
         else launch_lay_embed_rows(embed, d_ids, L.X, T, W, V, s);
-        const bool bf = !L.f32;
         auto norm_canon = [&](const float* nw_, const float* cw, size_t coff) {
             if (L.taps <= 0) { launch_lay_rms_rows(L.X, nullptr, nw_, L.Hc, T, W, cfg.eps, s); return; }
             if (all_decode) {
@@ -503,7 +541,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             g.A = L.Hc; g.lda = W; g.W = w.in_w; g.bias = w.in_b; g.C = L.P; g.ldc = w.in_rows; g.M = T; g.N = w.in_rows; g.K = W;
             g.act_split = w.g_off; g.act2 = LACT_SIGMOID;
             g.act = sp.mixer == LMIX_ATTN ? LACT_NONE : LACT_SILU;
-            launch_lgemm(g, bf, 1, s);
+            lay_gemm(*this, L, g, 1, s);
             int on = 0;
             const float* oa = nullptr;
             if (sp.mixer == LMIX_ATTN) {
@@ -532,7 +570,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             }
             LGemmArgs go;
             go.A = oa; go.lda = on; go.W = w.o_w; go.C = L.Y; go.ldc = W; go.M = T; go.N = W; go.K = on;
-            launch_lgemm(go, bf, 1, s);
+            lay_gemm(*this, L, go, 1, s);
             launch_lay_post_norm(L.X, L.Y, w.norm1b, L.mult, cfg.eps, T, W, nullptr, 0, s);
             if (sp.mlp != LMLP_NONE) {
                 norm_canon(w.norm2, w.canon2, w.c2_off);
@@ -540,10 +578,10 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     LGemmArgs gu;
                     gu.A = L.Hc; gu.lda = W; gu.W = w.gate; gu.W2 = w.up; gu.C = L.HH; gu.ldc = sp.ff; gu.M = T; gu.N = sp.ff; gu.K = W;
                     gu.act = LACT_GELU_TANH;
-                    launch_lgemm(gu, bf, 1, s);
+                    lay_gemm(*this, L, gu, 1, s);
                     LGemmArgs dn;
                     dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.C = L.Y; dn.ldc = W; dn.M = T; dn.N = W; dn.K = sp.ff;
-                    launch_lgemm(dn, bf, 1, s);
+                    lay_gemm(*this, L, dn, 1, s);
                     launch_lay_post_norm(L.X, L.Y, w.norm2b, L.mult, cfg.eps, T, W, nullptr, 0, s);
                 } else {
                     launch_lay_router(L.Hc, w.router, L.sel, L.wsel, T, W, sp.experts, sp.top, s);
@@ -552,11 +590,11 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     gu.A = L.Hc; gu.lda = W; gu.a_idx = L.srt; gu.a_div = sp.top;
                     gu.W = w.gate; gu.W2 = w.up; gu.w_stride = (size_t)sp.ff * W;
                     gu.C = L.HH; gu.ldc = sp.ff; gu.M = T; gu.N = sp.ff; gu.K = W; gu.grp_off = L.off; gu.act = LACT_SILU;
-                    launch_lgemm(gu, bf, sp.experts, s);
+                    lay_gemm(*this, L, gu, sp.experts, s);
                     LGemmArgs dn;
                     dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.w_stride = (size_t)W * sp.ff;
                     dn.C = L.YS; dn.ldc = W; dn.c_idx = L.srt; dn.M = T; dn.N = W; dn.K = sp.ff; dn.grp_off = L.off;
-                    launch_lgemm(dn, bf, sp.experts, s);
+                    lay_gemm(*this, L, dn, sp.experts, s);
                     launch_lay_post_norm(L.X, L.YS, w.norm2b, L.mult, cfg.eps, T, W, L.wsel, sp.top, s);
                 }
             }
@@ -573,7 +611,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             launch_lay_rms_rows(L.X, d_wrows + w0, L.final_norm, L.Xw, nr, W, cfg.eps, s);
             LGemmArgs hd;
             hd.A = L.Xw; hd.lda = W; hd.W = L.head; hd.C = logitsb; hd.ldc = V; hd.M = nr; hd.N = V; hd.K = W;
-            launch_lgemm(hd, bf, 1, s);
+            lay_gemm(*this, L, hd, 1, s);
             if (greedy_out) {
                 launch_lay_argmax_rows(logitsb, V, V, L.d_greedy, nr, s);
                 CM_HIP(hipMemcpyAsync(L.h_greedy, L.d_greedy, (size_t)nr * sizeof(uint32_t), hipMemcpyDeviceToHost, s));

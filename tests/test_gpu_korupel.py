@@ -352,3 +352,25 @@ def test_synthetic_registry_model_generates(tmp_path):
         assert m.decode_bytes_per_token(64) > m.weight_bytes() // 4
     finally:
         m.close()
+
+
+def test_bfloat16_products_on_the_shared_gemm_and_on_the_row_kernel_agree(tmp_path):
+    """Registry widths that fit the matrix-core GEMM of the other families (output widths of 128): a 100-token prompt (shared GEMM
+    for the products that fit), the same with the switch off (tiled kernel of this family), and token by token (row kernel)."""
+    from crane_amd import configs
+    cfg = configs.get_config("tiny-korupel")
+    P = U.random_weights(cfg, 15)
+    toks = U.tokens(100, cfg["vocab"], 15)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P, dtype="bfloat16")
+    try:
+        a, b, c = m.seq_alloc(), m.seq_alloc(), m.seq_alloc()
+        shared, _ = m.step_batch([(a, toks, _all(100))])
+        m.debug_set("lay_shared_gemm", 0)
+        tiled, _ = m.step_batch([(b, toks, _all(100))])
+        rows = np.concatenate([m.step_batch([(c, [t], [0])])[0] for t in toks])
+        for got in (shared, tiled, rows):
+            assert _err(got, want) < TOL_BF16
+        assert _err(shared, tiled) < TOL_BF16 and _err(rows, tiled) < TOL_BF16
+    finally:
+        m.close()
