@@ -558,8 +558,10 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
 #pragma unroll
     for (int c = 0; c < 16; ++c) acc[c] = 0.f;
     const size_t esz = KVT == KV_F32 ? 4 : 2;
-    for (long long v0 = 0; v0 < total; v0 += KT) {
-        __syncthreads();                   // previous tile fully consumed (and qs written, first time round)
+    const int nsplit = (int)gridDim.z;     // the visible keys' tiles are dealt round-robin to nsplit blocks (few queries, many keys)
+    __syncthreads();                       // qs written (a split may have no tile at all)
+    for (long long v0 = (long long)blockIdx.z * KT; v0 < total; v0 += (long long)KT * nsplit) {
+        __syncthreads();                   // previous tile fully consumed
         for (int rr = 0; rr < KT / 16; ++rr) {
             const int sl = qr + 16 * rr;
             const long long v = v0 + sl;
@@ -613,6 +615,16 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
             }
         }
     }
+    if (nsplit > 1) {                      // un-normalised partial sums + (running max, running sum) for the merge
+        const size_t pr = (((size_t)blockIdx.x * a.G + g) * nsplit + blockIdx.z) * LA_BQ + qr;
+        if (ln == 0) { a.part_ml[pr * 2] = m; a.part_ml[pr * 2 + 1] = l; }
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const int i = ln + 16 * c;
+            if (i < d) a.part_o[pr * d + i] = acc[c];
+        }
+        return;
+    }
     if (!qvalid) return;
     const float gate = a.proj[(size_t)row * a.ldp + a.g_off + head];
     const float inv = gate / l;
@@ -622,9 +634,44 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         if (i < d) a.out[(size_t)row * a.ldo + head * d + i] = acc[c] * inv;
     }
 }
+// merge of the splits of a tile: out = sum_z acc_z e^(m_z - M) / sum_z l_z e^(m_z - M) * gate
+__global__ __launch_bounds__(256) void lay_attn_merge_kernel(LAttnArgs a, int nsplit) {
+    const int2 tile = a.tiles[blockIdx.x];
+    const LaySegDev sg = a.segs[tile.x];
+    const int g = blockIdx.y, nrep = a.H / a.G, d = a.d;
+    const int q0 = tile.y, nq = min(LA_BQ, sg.n * nrep - q0);
+    const int qr = threadIdx.x >> 4, ln = threadIdx.x & 15;
+    if (qr >= nq) return;
+    const int qi = q0 + qr, lp = qi / nrep, head = g * nrep + (qi - lp * nrep), row = sg.row0 + lp;
+    const size_t p0 = (((size_t)blockIdx.x * a.G + g) * nsplit) * LA_BQ + qr;
+    float M = -INFINITY;
+    for (int z = 0; z < nsplit; ++z) M = fmaxf(M, a.part_ml[(p0 + (size_t)z * LA_BQ) * 2]);
+    float L = 0.f, acc[16];
+#pragma unroll
+    for (int c = 0; c < 16; ++c) acc[c] = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+        const size_t pr = p0 + (size_t)z * LA_BQ;
+        const float mz = a.part_ml[pr * 2];
+        if (mz == -INFINITY) continue;
+        const float w = expf(mz - M);
+        L = fmaf(a.part_ml[pr * 2 + 1], w, L);
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const int i = ln + 16 * c;
+            if (i < d) acc[c] = fmaf(a.part_o[pr * d + i], w, acc[c]);
+        }
+    }
+    const float inv = a.proj[(size_t)row * a.ldp + a.g_off + head] / L;
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+        const int i = ln + 16 * c;
+        if (i < d) a.out[(size_t)row * a.ldo + head * d + i] = acc[c] * inv;
+    }
+}
 void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s) {
     if (a.ntiles <= 0) return;
-    const dim3 grid((unsigned)a.ntiles, (unsigned)a.G);
+    const int nsplit = (a.part_o && a.part_ml && a.nsplit > 1) ? a.nsplit : 1;
+    const dim3 grid((unsigned)a.ntiles, (unsigned)a.G, (unsigned)nsplit);
     const bool narrow = a.d > 128;         // 32-key tiles keep the block inside 64 KiB of LDS up to d = 256
     const int KT = narrow ? 32 : 64;
     const size_t lds = (size_t)(LA_BQ * a.d + KT * (a.d + 1) + LA_BQ * KT) * sizeof(float);
@@ -635,6 +682,7 @@ void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s) {
         if (narrow) hipLaunchKernelGGL((lay_attn_kernel<KV_BF16, 32>), grid, dim3(256), lds, s, a);
         else hipLaunchKernelGGL((lay_attn_kernel<KV_BF16, 64>), grid, dim3(256), lds, s, a);
     }
+    if (nsplit > 1) hipLaunchKernelGGL(lay_attn_merge_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(256), 0, s, a, nsplit);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -709,8 +757,122 @@ __global__ __launch_bounds__(256) void lay_lightning_kernel(LLightArgs a, int C)
         if (j < ne) st[(size_t)i * e + j0 + j] = S[idx];
     }
 }
+// Long portions: the same recurrence in three launches that are parallel over chunks of LC tokens.
+//   1. every chunk's own contribution  U_c = sum_s decay^(n-1-s) k_s v_s^T                        (chunk, head, value slice)
+//   2. the states in front of the chunks by a scan over each sequence's chunks, in place: U_c <- S_c, S_(c+1) = decay^n S_c + U_c,
+//      last state back to the pool                                                              (sequence, head, state element)
+//   3. o_t = decay^(t+1) S_c^T q_t + sum_(s <= t) decay^(t-s) (q_t . k_s) v_s                      (chunk, head, value slice)
+// chunks[c] = {segment, first token of the chunk inside the portion}; a segment's chunks are consecutive, the first is segs[].pad0.
+constexpr int LC = 32;
+__global__ __launch_bounds__(256) void lay_light_chunk_kv_kernel(LLightArgs a) {
+    extern __shared__ float lds[];
+    const int d = a.d, e = a.e;
+    float* ks = lds;                       // [LC][d]
+    float* vs = ks + LC * d;               // [LC][ES]
+    float* pw = vs + LC * LL_ES;           // [LC + 1]
+    const int2 ch = a.chunks[blockIdx.x];
+    const LaySegDev sg = a.segs[ch.x];
+    const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
+    const int ne = min(LL_ES, e - j0), n = min(LC, sg.n - ch.y);
+    const float decay = a.decay[head];
+    if (tid <= LC) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
+    for (int idx = tid; idx < n * d; idx += 256) {
+        const int t = idx / d, i = idx - t * d;
+        ks[idx] = a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.k_off + (size_t)head * d + i];
+    }
+    for (int idx = tid; idx < n * LL_ES; idx += 256) {
+        const int t = idx / LL_ES, j = idx % LL_ES;
+        vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+    }
+    __syncthreads();
+    float* U = a.U + ((size_t)blockIdx.x * a.H + head) * d * e;
+    for (int idx = tid; idx < d * LL_ES; idx += 256) {
+        const int i = idx / LL_ES, j = idx % LL_ES;
+        float sv = 0.f;
+        for (int s = 0; s < n; ++s) sv = fmaf(pw[n - 1 - s] * ks[s * d + i], vs[s * LL_ES + j], sv);
+        if (j < ne) U[(size_t)i * e + j0 + j] = sv;
+    }
+}
+__global__ __launch_bounds__(256) void lay_light_scan_kernel(LLightArgs a) {
+    const LaySegDev sg = a.segs[blockIdx.x];
+    const int head = blockIdx.y, de = a.d * a.e;
+    const int el = blockIdx.z * 256 + threadIdx.x;
+    if (el >= de) return;
+    const float decay = a.decay[head];
+    const int nch = (sg.n + LC - 1) / LC;
+    const float pfull = powf(decay, (float)LC), plast = powf(decay, (float)(sg.n - (nch - 1) * LC));
+    float* st = a.state_pool + (size_t)sg.slot * a.slot_stride + a.st_off + (size_t)head * de + el;
+    float S = *st;
+    for (int c = 0; c < nch; ++c) {
+        float* u = a.U + ((size_t)(sg.pad0 + c) * a.H + head) * de + el;
+        const float own = *u;
+        *u = S;
+        S = fmaf(S, c == nch - 1 ? plast : pfull, own);
+    }
+    *st = S;
+}
+__global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) {
+    extern __shared__ float lds[];
+    const int d = a.d, e = a.e;
+    float* S = lds;                        // [d][ES] state in front of the chunk
+    float* qs = S + d * LL_ES;             // [LC][d]
+    float* ks = qs + LC * d;               // [LC][d]
+    float* vs = ks + LC * d;               // [LC][ES]
+    float* As = vs + LC * LL_ES;           // [LC][LC]
+    float* pw = As + LC * LC;              // [LC + 1]
+    const int2 ch = a.chunks[blockIdx.x];
+    const LaySegDev sg = a.segs[ch.x];
+    const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
+    const int ne = min(LL_ES, e - j0), n = min(LC, sg.n - ch.y);
+    const float decay = a.decay[head];
+    if (tid <= LC) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
+    const float* U = a.U + ((size_t)blockIdx.x * a.H + head) * d * e;
+    for (int idx = tid; idx < d * LL_ES; idx += 256) {
+        const int i = idx / LL_ES, j = idx % LL_ES;
+        S[idx] = j < ne ? U[(size_t)i * e + j0 + j] : 0.f;
+    }
+    for (int idx = tid; idx < n * d; idx += 256) {
+        const int t = idx / d, i = idx - t * d;
+        const size_t base = (size_t)(sg.row0 + ch.y + t) * a.ldp + (size_t)head * d + i;
+        qs[idx] = a.proj[base + a.q_off];
+        ks[idx] = a.proj[base + a.k_off];
+    }
+    for (int idx = tid; idx < n * LL_ES; idx += 256) {
+        const int t = idx / LL_ES, j = idx % LL_ES;
+        vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < n * n; idx += 256) {
+        const int t = idx / n, s = idx - t * n;
+        float dot = 0.f;
+        if (s <= t) {
+            for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * d + i], dot);
+            dot *= pw[t - s];
+        }
+        As[t * LC + s] = dot;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < n * LL_ES; idx += 256) {
+        const int t = idx / LL_ES, j = idx % LL_ES;
+        float inter = 0.f;
+        for (int i = 0; i < d; ++i) inter = fmaf(S[i * LL_ES + j], qs[t * d + i], inter);
+        float o = inter * pw[t + 1];
+        for (int s = 0; s <= t; ++s) o = fmaf(As[t * LC + s], vs[s * LL_ES + j], o);
+        if (j < ne) a.out[(size_t)(sg.row0 + ch.y + t) * a.ldo + (size_t)head * e + j0 + j] = o;
+    }
+}
+
 void launch_lay_lightning(const LLightArgs& a, hipStream_t s) {
     if (a.nseg <= 0) return;
+    if (a.U && a.chunks && a.nchunks > 0 && a.d <= 128) {
+        const dim3 gc((unsigned)a.nchunks, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES));
+        const size_t l1 = (size_t)(LC * a.d + LC * LL_ES + LC + 1) * sizeof(float);
+        const size_t l3 = (size_t)(a.d * LL_ES + 2 * LC * a.d + LC * LL_ES + LC * LC + LC + 1) * sizeof(float);
+        hipLaunchKernelGGL(lay_light_chunk_kv_kernel, gc, dim3(256), l1, s, a);
+        hipLaunchKernelGGL(lay_light_scan_kernel, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.d * a.e + 255) / 256)), dim3(256), 0, s, a);
+        hipLaunchKernelGGL(lay_light_chunk_out_kernel, gc, dim3(256), l3, s, a);
+        return;
+    }
     const int C = a.d > 128 ? 8 : 16;
     const size_t lds = (size_t)(a.d * LL_ES + 2 * C * a.d + C * LL_ES + C * C + C + 1) * sizeof(float);
     hipLaunchKernelGGL(lay_lightning_kernel, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES)), dim3(256), lds, s, a, C);
@@ -788,8 +950,43 @@ __global__ __launch_bounds__(256) void lay_argmax_rows_kernel(const float* __res
     }
     if (threadIdx.x == 0) out[blockIdx.x] = (uint32_t)(bi[0] == 0x7fffffff ? 0 : bi[0]);
 }
-void launch_lay_argmax_rows(const float* logits, int ld, int V, uint32_t* out, int n_rows, hipStream_t s) {
+// wide rows: LAY_ARGMAX_PARTS blocks per row leave (value, index) partials, one block per row picks among them
+__global__ __launch_bounds__(256) void lay_argmax_part_kernel(const float* __restrict__ logits, int ld, int V, float* __restrict__ pv,
+                                                              int* __restrict__ pi) {
+    __shared__ float bv[256];
+    __shared__ int bi[256];
+    const float* lr = logits + (size_t)blockIdx.x * ld;
+    const int per = (V + (int)gridDim.y - 1) / (int)gridDim.y, lo = blockIdx.y * per, hi = min(V, lo + per);
+    float best = -INFINITY; int idx = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += 256) { const float v = lr[i]; if (v > best) { best = v; idx = i; } }
+    bv[threadIdx.x] = best; bi[threadIdx.x] = idx;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) {
+        if ((int)threadIdx.x < st) {
+            const float ov = bv[threadIdx.x + st]; const int oi = bi[threadIdx.x + st];
+            if (ov > bv[threadIdx.x] || (ov == bv[threadIdx.x] && oi < bi[threadIdx.x])) { bv[threadIdx.x] = ov; bi[threadIdx.x] = oi; }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) { pv[blockIdx.x * gridDim.y + blockIdx.y] = bv[0]; pi[blockIdx.x * gridDim.y + blockIdx.y] = bi[0]; }
+}
+__global__ __launch_bounds__(64) void lay_argmax_final_kernel(const float* __restrict__ pv, const int* __restrict__ pi, int parts,
+                                                              uint32_t* __restrict__ out) {
+    if (threadIdx.x != 0) return;
+    float best = -INFINITY; int idx = 0x7fffffff;
+    for (int p = 0; p < parts; ++p) {
+        const float v = pv[blockIdx.x * parts + p]; const int i = pi[blockIdx.x * parts + p];
+        if (v > best || (v == best && i < idx)) { best = v; idx = i; }
+    }
+    out[blockIdx.x] = (uint32_t)(idx == 0x7fffffff ? 0 : idx);
+}
+void launch_lay_argmax_rows(const float* logits, int ld, int V, uint32_t* out, int n_rows, float* pv, int* pi, hipStream_t s) {
     if (n_rows <= 0) return;
+    if (pv && pi && V >= 8192) {
+        hipLaunchKernelGGL(lay_argmax_part_kernel, dim3((unsigned)n_rows, LAY_ARGMAX_PARTS), dim3(256), 0, s, logits, ld, V, pv, pi);
+        hipLaunchKernelGGL(lay_argmax_final_kernel, dim3((unsigned)n_rows), dim3(64), 0, s, pv, pi, LAY_ARGMAX_PARTS, out);
+        return;
+    }
     hipLaunchKernelGGL(lay_argmax_rows_kernel, dim3((unsigned)n_rows), dim3(256), 0, s, logits, ld, V, out);
 }
 

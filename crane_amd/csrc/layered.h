@@ -93,6 +93,9 @@ struct LAttnArgs {
     const float *r1, *r2;
     int H, G, d, page;
     float scale; long long win, keep;
+    // few query tiles, many keys (decode steps): nsplit blocks per tile share its key tiles and a merge launch follows;
+    // part_o [ntiles][G][nsplit][16][d], part_ml [ntiles][G][nsplit][16][2].  nsplit <= 1 or null scratch: one block per tile
+    int nsplit = 1; float* part_o = nullptr; float* part_ml = nullptr;
 };
 void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int kvt, const int32_t* bt, const LaySegDev* segs,
                          const int32_t* rowseg, int T, int G, int d, int page, hipStream_t s);
@@ -105,7 +108,11 @@ struct LLightArgs {
     const LaySegDev* segs; int nseg;
     const float* decay;
     int H, d, e;
+    // chunk-parallel form (long portions; head size up to 128): chunk table {segment, first token}, segs[].pad0 = a segment's first
+    // chunk, U = [nchunks][H][d][e] f32 scratch.  Null / 0: one block per (sequence, head, value slice) walks the portion.
+    float* U = nullptr; const int2* chunks = nullptr; int nchunks = 0;
 };
+constexpr int LAY_LIGHT_CHUNK = 32;
 void launch_lay_lightning(const LLightArgs& a, hipStream_t s);
 // out = o / rms(o) * w * gate over whole rows (gate already passed through the sigmoid)
 void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s);
@@ -114,6 +121,8 @@ void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float
 void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s);
 // counting sort of the T top (token, choice) pairs by expert: off [E + 1], srt [T top]
 void launch_lay_moe_plan(const int32_t* sel, int32_t* off, int32_t* srt, int n, int E, hipStream_t s);
-void launch_lay_argmax_rows(const float* logits, int ld, int V, uint32_t* out, int n_rows, hipStream_t s);
+constexpr int LAY_ARGMAX_PARTS = 64;
+// pv / pi: [n_rows][LAY_ARGMAX_PARTS] scratch of the two-launch form for wide rows (null: one block per row)
+void launch_lay_argmax_rows(const float* logits, int ld, int V, uint32_t* out, int n_rows, float* pv, int* pi, hipStream_t s);
 
 }  // namespace cm

@@ -41,6 +41,11 @@ struct Layered {
     bool shared_gemm = true;
     uint16_t* Abf = nullptr;           // [cap rounded up to 256][widest K] bf16 A operand
     float *G1 = nullptr, *G2 = nullptr;   // [cap][widest dense ff] the two products of a gated feed-forward
+    float* U = nullptr;                // lightning attention, chunk-parallel form: [chunks of a pass][widest H d e] f32
+    size_t u_stride = 0;
+    static constexpr int ATT_PARTS = 512;   // (query tile, key head, split) blocks of a split-key attention launch
+    float *att_po = nullptr, *att_pml = nullptr;
+    float* am_pv = nullptr; int* am_pi = nullptr;   // arg-max partials of the logits rows
     bool capture = false;              // cm_debug_set("lay_capture"): keep the residual stream after every layer of every pass
     std::vector<float> captured;
     ~Layered() {
@@ -386,6 +391,18 @@ void Model::alloc_runtime_layered() {
         if (dense_ff) { L.G1 = dalloc<float>(cap * (size_t)dense_ff); L.G2 = dalloc<float>(cap * (size_t)dense_ff); }
         ensure_gemm_workspace();
     }
+    size_t hde = 0; int max_d = 0;
+    for (const LayerSpec& sp : L.spec) {
+        if (sp.mixer == LMIX_LIGHTNING && sp.dim <= 128) hde = std::max(hde, (size_t)sp.heads * sp.dim * sp.vdim);
+        if (sp.mixer == LMIX_ATTN) max_d = std::max(max_d, sp.dim);
+    }
+    if (hde) { L.u_stride = hde; L.U = dalloc<float>((cap / LAY_LIGHT_CHUNK + (size_t)MAXB + 1) * hde); }
+    if (max_d) {
+        L.att_po = dalloc<float>((size_t)Layered::ATT_PARTS * 16 * max_d);
+        L.att_pml = dalloc<float>((size_t)Layered::ATT_PARTS * 16 * 2);
+    }
+    L.am_pv = dalloc<float>((size_t)Layered::LOGIT_ROWS * LAY_ARGMAX_PARTS);
+    L.am_pi = dalloc<int>((size_t)Layered::LOGIT_ROWS * LAY_ARGMAX_PARTS);
     L.Xw = dalloc<float>((size_t)Layered::LOGIT_ROWS * W);
     logitsb = dalloc<float>((size_t)Layered::LOGIT_ROWS * cfg.V);
     logits = dalloc<float>((size_t)cfg.V);
@@ -397,6 +414,7 @@ void Model::alloc_runtime_layered() {
     // one table upload per pass: ids | rowseg | wanted rows | segments | page tables | attention tiles per group size
     size_t tiles = 0;
     for (int nrep : L.nreps) tiles += 2 * (cap * (size_t)nrep / 16 + (size_t)MAXB + 1);
+    tiles += 2 * (cap / LAY_LIGHT_CHUNK + (size_t)MAXB + 1);      // lightning chunks
     L.tab_ints = 3 * cap + (size_t)MAXB * (sizeof(LaySegDev) / 4) + (size_t)MAXB * max_pages_per_seq + tiles + 64;
     L.d_tab = dalloc<int32_t>(L.tab_ints);
     CM_HIP(hipHostMalloc((void**)&L.h_tab, L.tab_ints * sizeof(int32_t)));
@@ -486,14 +504,18 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
         int32_t* t_wrows = tab + o; const size_t o_wrows = o; o += (size_t)T;
         LaySegDev* t_segs = (LaySegDev*)(tab + o); const size_t o_segs = o; o += (size_t)nseg * (sizeof(LaySegDev) / 4);
         int32_t* t_bt = tab + o; const size_t o_bt = o; o += (size_t)nseg * max_pages_per_seq;
-        int nw = 0, row = 0;
+        int nw = 0, row = 0, nchunks = 0, max_n = 0;
+        long long max_len = 0;
         bool all_decode = true;
         for (int k = 0; k < nseg; ++k) {
             const StepItem& it = items[ps[(size_t)k].item];
             Seq& q = seq(it.seq);
             const int n = ps[(size_t)k].n;
             const int sp = (int)q.len;
-            t_segs[k] = LaySegDev{row, n, sp, it.seq, k * max_pages_per_seq, 0, 0, 0};
+            t_segs[k] = LaySegDev{row, n, sp, it.seq, k * max_pages_per_seq, nchunks, 0, 0};
+            nchunks += (n + LAY_LIGHT_CHUNK - 1) / LAY_LIGHT_CHUNK;
+            max_n = std::max(max_n, n);
+            max_len = std::max(max_len, (long long)sp + n);
             memcpy(t_bt + (size_t)k * max_pages_per_seq, q.pages.data(), q.pages.size() * sizeof(int32_t));
             for (int r = 0; r < n; ++r) { t_ids[row + r] = (int32_t)it.ids[ps[(size_t)k].off + (size_t)r]; t_rowseg[row + r] = k; }
             if (it.n_want < 0) { if (ps[(size_t)k].off + (size_t)n == it.n) t_wrows[nw++] = row + n - 1; }
@@ -513,6 +535,11 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 for (int q0 = 0; q0 < t_segs[k].n * nrep; q0 += 16) { tab[o++] = k; tab[o++] = q0; ++cnt; }
             tiles[nrep] = {o_t, cnt};
         }
+        if (o & 1) ++o;
+        const size_t o_chunks = o;
+        if (L.U && max_n > LAY_LIGHT_CHUNK)
+            for (int k = 0; k < nseg; ++k)
+                for (int t0 = 0; t0 < t_segs[k].n; t0 += LAY_LIGHT_CHUNK) { tab[o++] = k; tab[o++] = t0; }
         if (o > L.tab_ints) throw CmError(CM_ERR_INVALID, "step tables overflow");
         CM_HIP(hipMemcpyAsync(L.d_tab, tab, o * sizeof(int32_t), hipMemcpyHostToDevice, s));
         const uint32_t* d_ids = (const uint32_t*)(L.d_tab + o_ids);
@@ -555,6 +582,12 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 a.tiles = (const int2*)(L.d_tab + tl.first); a.ntiles = tl.second;
                 a.r1 = w.r1; a.r2 = w.r2; a.H = sp.heads; a.G = sp.kv_heads; a.d = sp.dim; a.page = page;
                 a.scale = sp.scale; a.win = sp.win; a.keep = sp.keep;
+                {   // few query tiles and many visible keys (decode steps): share a tile's keys among blocks
+                    const long long seen = std::min<long long>(max_len, sp.win + sp.keep);
+                    const int key_tiles = (int)((seen + 63) / 64), blocks = std::max(1, a.ntiles * sp.kv_heads);
+                    a.nsplit = std::max(1, std::min({16, key_tiles / 2, 256 / blocks, Layered::ATT_PARTS / blocks}));
+                    a.part_o = L.att_po; a.part_ml = L.att_pml;
+                }
                 launch_lay_attn(a, kv_mode, s);
                 on = sp.heads * sp.dim; oa = L.O;
             } else {
@@ -563,6 +596,9 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 a.out = L.O; a.ldo = sp.heads * sp.vdim;
                 a.state_pool = state_pool; a.slot_stride = state_slot_elems; a.st_off = w.st_off;
                 a.segs = d_segs; a.nseg = nseg; a.decay = w.decay; a.H = sp.heads; a.d = sp.dim; a.e = sp.vdim;
+                if (L.U && max_n > LAY_LIGHT_CHUNK && sp.dim <= 128) {       // a long portion in the pass: parallel over chunks
+                    a.U = L.U; a.chunks = (const int2*)(L.d_tab + o_chunks); a.nchunks = nchunks;
+                }
                 launch_lay_lightning(a, s);
                 on = sp.heads * sp.vdim;
                 launch_lay_rms_gate(L.O, L.P + w.g_off, w.in_rows, w.mix_norm, L.O2, T, on, cfg.eps, s);
@@ -613,7 +649,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             hd.A = L.Xw; hd.lda = W; hd.W = L.head; hd.C = logitsb; hd.ldc = V; hd.M = nr; hd.N = V; hd.K = W;
             lay_gemm(*this, L, hd, 1, s);
             if (greedy_out) {
-                launch_lay_argmax_rows(logitsb, V, V, L.d_greedy, nr, s);
+                launch_lay_argmax_rows(logitsb, V, V, L.d_greedy, nr, L.am_pv, L.am_pi, s);
                 CM_HIP(hipMemcpyAsync(L.h_greedy, L.d_greedy, (size_t)nr * sizeof(uint32_t), hipMemcpyDeviceToHost, s));
             }
             if (logits_out) CM_HIP(hipMemcpyAsync(L.h_rows, logitsb, (size_t)nr * V * sizeof(float), hipMemcpyDeviceToHost, s));

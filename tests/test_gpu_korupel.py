@@ -374,3 +374,23 @@ def test_bfloat16_products_on_the_shared_gemm_and_on_the_row_kernel_agree(tmp_pa
         assert _err(shared, tiled) < TOL_BF16 and _err(rows, tiled) < TOL_BF16
     finally:
         m.close()
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", TOL_F32), ("bfloat16", TOL_BF16)])
+def test_decode_steps_over_hundreds_of_keys_and_a_long_portion_in_chunks(tmp_path, dtype, tol):
+    """A window of hundreds of positions: decode steps deal the key tiles of a query tile to several blocks and merge them; the
+    long portion in front runs the lightning layer parallel over chunks (the state in front of every chunk by a scan)."""
+    cfg = U.config([U.layer("attention", U.DENSE, **U.attn(heads=4, kv_heads=2, dim=16, size=300, keep_first=5)),
+                    U.layer("lightning", None, **U.light(heads=2, dim=16, vdim=40, decay=(0.9, 0.999)))], vocab=71, width=48)
+    P = U.random_weights(cfg, 16)
+    toks = U.tokens(430, cfg["vocab"], 16)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P, dtype=dtype)
+    try:
+        s = m.seq_alloc()
+        first, _ = m.step_batch([(s, toks[:395], [0, 31, 32, 33, 200, 394])])
+        assert _err(first, want[[0, 31, 32, 33, 200, 394]]) < tol
+        got = np.concatenate([m.step_batch([(s, [t], [0])])[0] for t in toks[395:]])
+        assert _err(got, want[395:]) < tol
+    finally:
+        m.close()
