@@ -569,6 +569,14 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
                 const long long j = v < sink_hi ? v : main_lo + (v - sink_hi);
                 const int pg = a.bt[sg.bt_off + (int)(j / a.page)];
                 const char* src = (const char*)a.kpool + ((((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * d) * esz;
+                if (KVT != KV_F32 && (d & 7) == 0) {             // 16 bytes = 8 cached keys per lane and load
+                    for (int i = ln * 8; i < d; i += 128) {
+                        const u32x4 p = *(const u32x4*)((const uint16_t*)src + i);
+                        float* dst = ks + sl * ldk + i;
+                        dst[0] = bf16_lo(p.x); dst[1] = bf16_hi(p.x); dst[2] = bf16_lo(p.y); dst[3] = bf16_hi(p.y);
+                        dst[4] = bf16_lo(p.z); dst[5] = bf16_hi(p.z); dst[6] = bf16_lo(p.w); dst[7] = bf16_hi(p.w);
+                    }
+                } else
                 for (int i = ln; i < d; i += 16)
                     ks[sl * ldk + i] = KVT == KV_F32 ? ((const float*)src)[i] : bf16_to_f32(((const uint16_t*)src)[i]);
             } else {
@@ -862,8 +870,48 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
     }
 }
 
+// single-token portions (decode steps): S <- decay S + k v^T and o = S^T q straight on the state in HBM, no staging; thread =
+// (value column j, 1/8 of the key rows); the eight partial sums of a column meet in LDS
+__global__ __launch_bounds__(256) void lay_light_decode_kernel(LLightArgs a) {
+    __shared__ float qk[2 * 256];
+    __shared__ float part[8][LL_ES];
+    const int d = a.d, e = a.e;
+    const LaySegDev sg = a.segs[blockIdx.x];
+    const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
+    const int j = tid & (LL_ES - 1), rg = tid >> 5;
+    const float decay = a.decay[head];
+    const size_t prow = (size_t)sg.row0 * a.ldp;
+    for (int i = tid; i < d; i += 256) {
+        qk[i] = a.proj[prow + a.q_off + (size_t)head * d + i];
+        qk[256 + i] = a.proj[prow + a.k_off + (size_t)head * d + i];
+    }
+    __syncthreads();
+    const bool ok = j0 + j < e;
+    const float v = ok ? a.proj[prow + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+    float* st = a.state_pool + (size_t)sg.slot * a.slot_stride + a.st_off + (size_t)head * d * e + j0 + j;
+    float o = 0.f;
+    if (ok)
+        for (int i = rg; i < d; i += 8) {
+            const float sv = fmaf(st[(size_t)i * e], decay, qk[256 + i] * v);
+            st[(size_t)i * e] = sv;
+            o = fmaf(sv, qk[i], o);
+        }
+    part[rg][j] = o;
+    __syncthreads();
+    if (rg == 0 && ok) {
+        float t = 0.f;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) t += part[r][j];
+        a.out[(size_t)sg.row0 * a.ldo + (size_t)head * e + j0 + j] = t;
+    }
+}
+
 void launch_lay_lightning(const LLightArgs& a, hipStream_t s) {
     if (a.nseg <= 0) return;
+    if (a.all_single && a.d <= 256) {
+        hipLaunchKernelGGL(lay_light_decode_kernel, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES)), dim3(256), 0, s, a);
+        return;
+    }
     if (a.U && a.chunks && a.nchunks > 0 && a.d <= 128) {
         const dim3 gc((unsigned)a.nchunks, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES));
         const size_t l1 = (size_t)(LC * a.d + LC * LL_ES + LC + 1) * sizeof(float);

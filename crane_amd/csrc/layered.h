@@ -111,6 +111,7 @@ struct LLightArgs {
     // chunk-parallel form (long portions; head size up to 128): chunk table {segment, first token}, segs[].pad0 = a segment's first
     // chunk, U = [nchunks][H][d][e] f32 scratch.  Null / 0: one block per (sequence, head, value slice) walks the portion.
     float* U = nullptr; const int2* chunks = nullptr; int nchunks = 0;
+    bool all_single = false;     // every portion of the pass is one token (decode steps): the state is updated in place in HBM
 };
 constexpr int LAY_LIGHT_CHUNK = 32;
 void launch_lay_lightning(const LLightArgs& a, hipStream_t s);

@@ -585,7 +585,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 {   // few query tiles and many visible keys (decode steps): share a tile's keys among blocks
                     const long long seen = std::min<long long>(max_len, sp.win + sp.keep);
                     const int key_tiles = (int)((seen + 63) / 64), blocks = std::max(1, a.ntiles * sp.kv_heads);
-                    a.nsplit = std::max(1, std::min({16, key_tiles / 2, 256 / blocks, Layered::ATT_PARTS / blocks}));
+                    a.nsplit = std::max(1, std::min({32, key_tiles, 256 / blocks, Layered::ATT_PARTS / blocks}));
                     a.part_o = L.att_po; a.part_ml = L.att_pml;
                 }
                 launch_lay_attn(a, kv_mode, s);
@@ -596,6 +596,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 a.out = L.O; a.ldo = sp.heads * sp.vdim;
                 a.state_pool = state_pool; a.slot_stride = state_slot_elems; a.st_off = w.st_off;
                 a.segs = d_segs; a.nseg = nseg; a.decay = w.decay; a.H = sp.heads; a.d = sp.dim; a.e = sp.vdim;
+                a.all_single = all_decode;
                 if (L.U && max_n > LAY_LIGHT_CHUNK && sp.dim <= 128) {       // a long portion in the pass: parallel over chunks
                     a.U = L.U; a.chunks = (const int2*)(L.d_tab + o_chunks); a.nchunks = nchunks;
                 }
