@@ -185,6 +185,65 @@ __global__ __launch_bounds__(256) void lay_norm_canon_decode_kernel(const float*
         out[(size_t)sg.row0 * W + c] = acc;
     }
 }
+// decode rows: the residual update of the sublayer that just finished AND the norm + convolution in front of the next one, one
+// launch: x += mult * RMSNorm(y) * pw (y as in lay_post_norm_kernel), then as lay_norm_canon_decode_kernel on the new x
+__global__ __launch_bounds__(256) void lay_post_norm_canon_decode_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                                         const float* __restrict__ pw, float mult, const float* __restrict__ wsel,
+                                                                         int top, const float* __restrict__ nw, float eps, float* __restrict__ out,
+                                                                         const float* __restrict__ cw, float* __restrict__ conv_pool,
+                                                                         size_t slot_stride, size_t off, const LaySegDev* __restrict__ segs, int W,
+                                                                         int taps) {
+    __shared__ float red[4];
+    const LaySegDev sg = segs[blockIdx.x];
+    const int r = sg.row0;
+    float* xr = x + (size_t)r * W;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float v;
+        if (wsel) {
+            v = 0.f;
+            for (int k = 0; k < top; ++k) v += wsel[(size_t)r * top + k] * y[((size_t)r * top + k) * W + c];
+        } else v = y[(size_t)r * W + c];
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float rsy = 1.f / sqrtf(ss / (float)W + eps);
+    float sx = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float v;
+        if (wsel) {
+            v = 0.f;
+            for (int k = 0; k < top; ++k) v += wsel[(size_t)r * top + k] * y[((size_t)r * top + k) * W + c];
+        } else v = y[(size_t)r * W + c];
+        const float xn = xr[c] + mult * (v * rsy * pw[c]);
+        xr[c] = xn;                        // read back below by the same thread
+        sx += xn * xn;
+    }
+    sx = block_sum(sx, red);
+    const float rs = 1.f / sqrtf(sx / (float)W + eps);
+    float* tail = conv_pool + (size_t)sg.slot * slot_stride + off;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float hv = xr[c] * rs * nw[c];
+        float acc = hv;
+        if (taps > 0) {
+            acc += cw[(size_t)c * taps + (taps - 1)] * hv;
+            for (int j = 0; j < taps - 1; ++j) {
+                const float tv = tail[(size_t)j * W + c];
+                acc += cw[(size_t)c * taps + j] * tv;
+                if (j > 0) tail[(size_t)(j - 1) * W + c] = tv;
+            }
+            if (taps > 1) tail[(size_t)(taps - 2) * W + c] = hv;
+        }
+        out[(size_t)r * W + c] = acc;
+    }
+}
+void launch_lay_post_norm_canon_decode(float* x, const float* y, const float* pw, float mult, const float* wsel, int top, const float* nw,
+                                       float eps, float* out, const float* cw, float* conv_pool, size_t slot_stride, size_t off,
+                                       const LaySegDev* segs, int T, int W, int taps, hipStream_t s) {
+    if (T <= 0) return;
+    hipLaunchKernelGGL(lay_post_norm_canon_decode_kernel, dim3((unsigned)T), dim3(256), 0, s, x, y, pw, mult, wsel, top, nw, eps, out, cw,
+                       conv_pool, slot_stride, off, segs, W, taps);
+}
 void launch_lay_norm_canon_decode(const float* x, const float* nw, float eps, float* out, const float* cw, float* conv_pool,
                                   size_t slot_stride, size_t off, const LaySegDev* segs, int T, int W, int taps, hipStream_t s) {
     if (T <= 0) return;

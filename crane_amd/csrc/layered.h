@@ -81,6 +81,10 @@ void launch_lay_canon_tail(const float* h, float* conv_pool, size_t slot_stride,
 // single-token rows only (every segment n = 1): RMS norm, convolution and tail shift in one launch
 void launch_lay_norm_canon_decode(const float* x, const float* nw, float eps, float* out, const float* cw, float* conv_pool,
                                   size_t slot_stride, size_t off, const LaySegDev* segs, int T, int W, int taps, hipStream_t s);
+// single-token rows only: lay_post_norm of the finished sublayer and lay_norm_canon_decode of the next one in one launch
+void launch_lay_post_norm_canon_decode(float* x, const float* y, const float* pw, float mult, const float* wsel, int top, const float* nw,
+                                       float eps, float* out, const float* cw, float* conv_pool, size_t slot_stride, size_t off,
+                                       const LaySegDev* segs, int T, int W, int taps, hipStream_t s);
 // x += mult * RMSNorm(y) * w;  sel != null: y[r] = sum_k wsel[r top + k] * ys[r top + k] (mixture-of-experts combine)
 void launch_lay_post_norm(float* x, const float* y, const float* w, float mult, float eps, int T, int W, const float* wsel, int top,
                           hipStream_t s);

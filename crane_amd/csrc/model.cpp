@@ -775,8 +775,7 @@ void Model::cow_page(int s, size_t idx) {
     q.pages[idx] = newp;
     if (layered) { layered_cow_page(oldp, newp); if (active_seq == s) active_pages_uploaded = std::min(active_pages_uploaded, idx); return; }
     const size_t pitch = (size_t)n_pages * page_bytes;
-    // one plain copy per (layer, K | V) plane of the pool (a pitched 2-D copy of the same bytes was the first call of two test
-    // runs that ended with a device error on the GPU boxes; plain device-to-device copies are what the other paths use)
+    // one plain copy per (layer, K | V) plane of the pool
     for (size_t pl = 0; pl < (size_t)n_kv_layers * 2; ++pl)
         CM_HIP(hipMemcpyAsync(kv_pool + pl * pitch + (size_t)newp * page_bytes, kv_pool + pl * pitch + (size_t)oldp * page_bytes,
                               page_bytes, hipMemcpyDeviceToDevice, stream));
@@ -1529,6 +1528,7 @@ void Model::prefill_multi(const int32_t* sq, const uint32_t* const* ids, const s
         Seq& q = seq(sq[i]);
         memcpy(h_ids + row, ids[i], lens[i] * sizeof(uint32_t));
         memcpy(h_btb + i * (size_t)max_pages_per_seq, q.pages.data(), q.pages.size() * sizeof(int32_t));
+        for (size_t pz = q.pages.size(); pz < (size_t)max_pages_per_seq; ++pz) h_btb[i * (size_t)max_pages_per_seq + pz] = 0;
         segs[i] = PrefillSeg{row, (int)lens[i], 0, sq[i], 0, d_btb + i * (size_t)max_pages_per_seq};
         StepState& hs = h_stb[i];
         memset(&hs, 0, sizeof hs);
@@ -1762,6 +1762,10 @@ void Model::ensure_batch_buffers() {
     lm_gridb = g;
     CM_HIP(hipHostMalloc((void**)&h_stb, MAXB * sizeof(StepState)));
     CM_HIP(hipHostMalloc((void**)&h_btb, (size_t)MAXB * max_pages_per_seq * sizeof(int32_t)));
+    // whole rows of this mirror are uploaded, and the decode attention requests the K / V rows of its first chunks before it knows
+    // the sequence's length (speculative loads, clamped to the table's width only): entries past a sequence's pages must be valid
+    // page ids -- pinned memory is not zero when the allocator hands back a block an earlier handle freed
+    memset(h_btb, 0, (size_t)MAXB * max_pages_per_seq * sizeof(int32_t));
     CM_HIP(hipHostMalloc((void**)&h_logitsb, (size_t)MAXB * cfg.V * sizeof(float)));
     CM_HIP(hipMemsetAsync(d_btb, 0, (size_t)MAXB * max_pages_per_seq * sizeof(int32_t), stream));
 }
@@ -1848,6 +1852,7 @@ void Model::decode_batch(const int32_t* sq, const uint32_t* toks, size_t n, floa
             memset(&hs, 0, sizeof hs);
             hs.token = toks[g0 + b]; hs.pos = (int32_t)q.len; hs.slot = sidx; hs.rsv[0] = q.rope_delta;
             memcpy(h_btb + (size_t)b * max_pages_per_seq, q.pages.data(), q.pages.size() * sizeof(int32_t));
+            for (size_t pz = q.pages.size(); pz < (size_t)max_pages_per_seq; ++pz) h_btb[(size_t)b * max_pages_per_seq + pz] = 0;
         }
         CM_HIP(hipMemcpyAsync(stb, h_stb, (size_t)nb * sizeof(StepState), hipMemcpyHostToDevice, s));
         CM_HIP(hipMemcpyAsync(d_btb, h_btb, (size_t)nb * max_pages_per_seq * sizeof(int32_t), hipMemcpyHostToDevice, s));

@@ -517,6 +517,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             max_n = std::max(max_n, n);
             max_len = std::max(max_len, (long long)sp + n);
             memcpy(t_bt + (size_t)k * max_pages_per_seq, q.pages.data(), q.pages.size() * sizeof(int32_t));
+            for (size_t pz = q.pages.size(); pz < (size_t)max_pages_per_seq; ++pz) t_bt[(size_t)k * max_pages_per_seq + pz] = 0;
             for (int r = 0; r < n; ++r) { t_ids[row + r] = (int32_t)it.ids[ps[(size_t)k].off + (size_t)r]; t_rowseg[row + r] = k; }
             if (it.n_want < 0) { if (ps[(size_t)k].off + (size_t)n == it.n) t_wrows[nw++] = row + n - 1; }
             else for (int j = 0; j < it.n_want; ++j) {
@@ -550,7 +551,24 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
 
         if (W % 4 == 0) launch_embed_rows(embed, d_ids, L.X, T, W, V, s);
         else launch_lay_embed_rows(embed, d_ids, L.X, T, W, V, s);
+        // the residual update of a finished sublayer waits for the next norm: decode steps run both in one launch
+        struct { const float* y = nullptr; const float* w = nullptr; const float* wsel = nullptr; int top = 0; } pend;
+        auto flush_post = [&]() {
+            if (pend.y) launch_lay_post_norm(L.X, pend.y, pend.w, L.mult, cfg.eps, T, W, pend.wsel, pend.top, s);
+            pend.y = nullptr;
+        };
+        auto post_norm = [&](const float* y, const float* w_, const float* wsel, int top) {
+            flush_post();
+            pend.y = y; pend.w = w_; pend.wsel = wsel; pend.top = top;
+        };
         auto norm_canon = [&](const float* nw_, const float* cw, size_t coff) {
+            if (pend.y && all_decode) {
+                launch_lay_post_norm_canon_decode(L.X, pend.y, pend.w, L.mult, pend.wsel, pend.top, nw_, cfg.eps, L.Hc, cw, conv_pool,
+                                                  conv_slot_elems, coff, d_segs, T, W, L.taps, s);
+                pend.y = nullptr;
+                return;
+            }
+            flush_post();
             if (L.taps <= 0) { launch_lay_rms_rows(L.X, nullptr, nw_, L.Hc, T, W, cfg.eps, s); return; }
             if (all_decode) {
                 launch_lay_norm_canon_decode(L.X, nw_, cfg.eps, L.Hc, cw, conv_pool, conv_slot_elems, coff, d_segs, T, W, L.taps, s);
@@ -608,7 +626,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             LGemmArgs go;
             go.A = oa; go.lda = on; go.W = w.o_w; go.C = L.Y; go.ldc = W; go.M = T; go.N = W; go.K = on;
             lay_gemm(*this, L, go, 1, s);
-            launch_lay_post_norm(L.X, L.Y, w.norm1b, L.mult, cfg.eps, T, W, nullptr, 0, s);
+            post_norm(L.Y, w.norm1b, nullptr, 0);
             if (sp.mlp != LMLP_NONE) {
                 norm_canon(w.norm2, w.canon2, w.c2_off);
                 if (sp.mlp == LMLP_DENSE) {
@@ -619,7 +637,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     LGemmArgs dn;
                     dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.C = L.Y; dn.ldc = W; dn.M = T; dn.N = W; dn.K = sp.ff;
                     lay_gemm(*this, L, dn, 1, s);
-                    launch_lay_post_norm(L.X, L.Y, w.norm2b, L.mult, cfg.eps, T, W, nullptr, 0, s);
+                    post_norm(L.Y, w.norm2b, nullptr, 0);
                 } else {
                     launch_lay_router(L.Hc, w.router, L.sel, L.wsel, T, W, sp.experts, sp.top, s);
                     launch_lay_moe_plan(L.sel, L.off, L.srt, T * sp.top, sp.experts, s);
@@ -632,9 +650,10 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.w_stride = (size_t)W * sp.ff;
                     dn.C = L.YS; dn.ldc = W; dn.c_idx = L.srt; dn.M = T; dn.N = W; dn.K = sp.ff; dn.grp_off = L.off;
                     lay_gemm(*this, L, dn, sp.experts, s);
-                    launch_lay_post_norm(L.X, L.YS, w.norm2b, L.mult, cfg.eps, T, W, L.wsel, sp.top, s);
+                    post_norm(L.YS, w.norm2b, L.wsel, sp.top);
                 }
             }
+            if (L.capture || li + 1 == L.spec.size()) flush_post();
             if (L.capture) {
                 const size_t at = L.captured.size();
                 L.captured.resize(at + (size_t)T * W);
