@@ -646,12 +646,18 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         float sc[KT / 16];
         float tmax = -INFINITY;
 #pragma unroll
+        for (int c = 0; c < KT / 16; ++c) sc[c] = 0.f;
+        for (int i = 0; i < d; ++i) {          // one read of q per KT / 16 keys
+            const float qv = qs[qr * d + i];
+#pragma unroll
+            for (int c = 0; c < KT / 16; ++c) sc[c] = fmaf(qv, ks[(ln + 16 * c) * ldk + i], sc[c]);
+        }
+#pragma unroll
         for (int c = 0; c < KT / 16; ++c) {
             const int sl = ln + 16 * c;
             const long long v = v0 + sl;
             const long long j = v < sink_hi ? v : main_lo + (v - sink_hi);
-            float dot = 0.f;
-            for (int i = 0; i < d; ++i) dot = fmaf(qs[qr * d + i], ks[sl * ldk + i], dot);
+            const float dot = sc[c];
             const long long dist = pos - j;
             const bool vis = qvalid && v < total && dist >= 0 && (dist < a.win || j < a.keep);
             sc[c] = vis ? dot * a.scale - r1 * log1pf(r2 * (float)dist) : -INFINITY;
@@ -673,12 +679,13 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         __syncthreads();
         const int kn = (int)min((long long)KT, total - v0);
 #pragma unroll
-        for (int c = 0; c < 16; ++c) {
-            const int i = ln + 16 * c;
-            if (i < d) {
-                float o = acc[c] * corr;
-                for (int sl = 0; sl < kn; ++sl) o = fmaf(ps[qr * KT + sl], ks[sl * ldk + i], o);
-                acc[c] = o;
+        for (int c = 0; c < 16; ++c) acc[c] *= corr;
+        for (int sl = 0; sl < kn; ++sl) {      // one read of the weight per d / 16 value elements
+            const float p = ps[qr * KT + sl];
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                const int i = ln + 16 * c;
+                if (i < d) acc[c] = fmaf(p, ks[sl * ldk + i], acc[c]);
             }
         }
     }
@@ -883,8 +890,9 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
     const int d = a.d, e = a.e;
     float* S = lds;                        // [d][ES] state in front of the chunk
     float* qs = S + d * LL_ES;             // [LC][d]
-    float* ks = qs + LC * d;               // [LC][d]
-    float* vs = ks + LC * d;               // [LC][ES]
+    const int ldk = d + 1;                 // a wave's lanes read 32 different key rows at once: odd stride, no bank conflicts
+    float* ks = qs + LC * d;               // [LC][d + 1]
+    float* vs = ks + LC * ldk;             // [LC][ES]
     float* As = vs + LC * LL_ES;           // [LC][LC]
     float* pw = As + LC * LC;              // [LC + 1]
     const int2 ch = a.chunks[blockIdx.x];
@@ -902,7 +910,7 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
         const int t = idx / d, i = idx - t * d;
         const size_t base = (size_t)(sg.row0 + ch.y + t) * a.ldp + (size_t)head * d + i;
         qs[idx] = a.proj[base + a.q_off];
-        ks[idx] = a.proj[base + a.k_off];
+        ks[t * ldk + i] = a.proj[base + a.k_off];
     }
     for (int idx = tid; idx < n * LL_ES; idx += 256) {
         const int t = idx / LL_ES, j = idx % LL_ES;
@@ -913,7 +921,7 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
         const int t = idx / n, s = idx - t * n;
         float dot = 0.f;
         if (s <= t) {
-            for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * d + i], dot);
+            for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * ldk + i], dot);
             dot *= pw[t - s];
         }
         As[t * LC + s] = dot;
@@ -974,7 +982,7 @@ void launch_lay_lightning(const LLightArgs& a, hipStream_t s) {
     if (a.U && a.chunks && a.nchunks > 0 && a.d <= 128) {
         const dim3 gc((unsigned)a.nchunks, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES));
         const size_t l1 = (size_t)(LC * a.d + LC * LL_ES + LC + 1) * sizeof(float);
-        const size_t l3 = (size_t)(a.d * LL_ES + 2 * LC * a.d + LC * LL_ES + LC * LC + LC + 1) * sizeof(float);
+        const size_t l3 = (size_t)(a.d * LL_ES + 2 * LC * a.d + LC + LC * LL_ES + LC * LC + LC + 1) * sizeof(float);
         hipLaunchKernelGGL(lay_light_chunk_kv_kernel, gc, dim3(256), l1, s, a);
         hipLaunchKernelGGL(lay_light_scan_kernel, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.d * a.e + 255) / 256)), dim3(256), 0, s, a);
         hipLaunchKernelGGL(lay_light_chunk_out_kernel, gc, dim3(256), l3, s, a);
