@@ -237,10 +237,82 @@ __global__ __launch_bounds__(256) void lay_post_norm_canon_decode_kernel(float* 
         out[(size_t)r * W + c] = acc;
     }
 }
+// the same for rows of up to 256 EPT channels: every operand of a channel is requested up front and lives in registers, so the
+// launch costs two block reductions instead of three dependent sweeps over memory
+template <int EPT>
+__global__ __launch_bounds__(256) void lay_post_norm_canon_decode_reg_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                                             const float* __restrict__ pw, float mult,
+                                                                             const float* __restrict__ wsel, int top,
+                                                                             const float* __restrict__ nw, float eps, float* __restrict__ out,
+                                                                             const float* __restrict__ cw, float* __restrict__ conv_pool,
+                                                                             size_t slot_stride, size_t off, const LaySegDev* __restrict__ segs,
+                                                                             int W, int taps) {
+    __shared__ float red[4];
+    const LaySegDev sg = segs[blockIdx.x];
+    const int r = sg.row0;
+    float* xr = x + (size_t)r * W;
+    float yv[EPT], xv[EPT], pv[EPT], nv[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+        const int c = threadIdx.x + 256 * e;
+        const bool ok = c < W;
+        float v = 0.f;
+        if (ok) {
+            if (wsel) { for (int k = 0; k < top; ++k) v += wsel[(size_t)r * top + k] * y[((size_t)r * top + k) * W + c]; }
+            else v = y[(size_t)r * W + c];
+        }
+        yv[e] = v;
+        xv[e] = ok ? xr[c] : 0.f;
+        pv[e] = ok ? pw[c] : 0.f;
+        nv[e] = ok ? nw[c] : 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) ss += yv[e] * yv[e];
+    ss = block_sum(ss, red);
+    const float rsy = 1.f / sqrtf(ss / (float)W + eps);
+    float sx = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+        xv[e] += mult * (yv[e] * rsy * pv[e]);
+        sx += xv[e] * xv[e];
+    }
+    sx = block_sum(sx, red);
+    const float rs = 1.f / sqrtf(sx / (float)W + eps);
+    float* tail = conv_pool + (size_t)sg.slot * slot_stride + off;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+        const int c = threadIdx.x + 256 * e;
+        if (c >= W) continue;
+        xr[c] = xv[e];
+        const float hv = xv[e] * rs * nv[e];
+        float acc = hv;
+        if (taps > 0) {
+            acc += cw[(size_t)c * taps + (taps - 1)] * hv;
+            for (int j = 0; j < taps - 1; ++j) {
+                const float tv = tail[(size_t)j * W + c];
+                acc += cw[(size_t)c * taps + j] * tv;
+                if (j > 0) tail[(size_t)(j - 1) * W + c] = tv;
+            }
+            if (taps > 1) tail[(size_t)(taps - 2) * W + c] = hv;
+        }
+        out[(size_t)r * W + c] = acc;
+    }
+}
 void launch_lay_post_norm_canon_decode(float* x, const float* y, const float* pw, float mult, const float* wsel, int top, const float* nw,
                                        float eps, float* out, const float* cw, float* conv_pool, size_t slot_stride, size_t off,
                                        const LaySegDev* segs, int T, int W, int taps, hipStream_t s) {
     if (T <= 0) return;
+    if (W <= 1024) {
+        hipLaunchKernelGGL(lay_post_norm_canon_decode_reg_kernel<4>, dim3((unsigned)T), dim3(256), 0, s, x, y, pw, mult, wsel, top, nw, eps, out,
+                           cw, conv_pool, slot_stride, off, segs, W, taps);
+        return;
+    }
+    if (W <= 4096) {
+        hipLaunchKernelGGL(lay_post_norm_canon_decode_reg_kernel<16>, dim3((unsigned)T), dim3(256), 0, s, x, y, pw, mult, wsel, top, nw, eps, out,
+                           cw, conv_pool, slot_stride, off, segs, W, taps);
+        return;
+    }
     hipLaunchKernelGGL(lay_post_norm_canon_decode_kernel, dim3((unsigned)T), dim3(256), 0, s, x, y, pw, mult, wsel, top, nw, eps, out, cw,
                        conv_pool, slot_stride, off, segs, W, taps);
 }
@@ -605,13 +677,14 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
     const bool qvalid = qr < nq;
     const int qi = q0 + (qvalid ? qr : 0);
     const int lp = qi / nrep, head = g * nrep + (qi - lp * nrep);
-    const long long pos = (long long)sg.start_pos + lp;
+    const int pos = sg.start_pos + lp;
     const int row = sg.row0 + lp;
+    const int win = (int)min(a.win, 1ll << 30), keep = (int)min(a.keep, 1ll << 30);
     for (int i = ln; i < d; i += 16) qs[qr * d + i] = qvalid ? a.proj[(size_t)row * a.ldp + a.q_off + head * d + i] : 0.f;
-    const long long pmin = (long long)sg.start_pos + q0 / nrep, pmax = (long long)sg.start_pos + (q0 + nq - 1) / nrep;
-    const long long main_lo = max(0ll, pmin - a.win + 1);
-    const long long sink_hi = min(a.keep, main_lo);
-    const long long total = sink_hi + (pmax - main_lo + 1);
+    const int pmin = sg.start_pos + q0 / nrep, pmax = sg.start_pos + (q0 + nq - 1) / nrep;
+    const int main_lo = max(0, pmin - win + 1);
+    const int sink_hi = min(keep, main_lo);
+    const int total = sink_hi + (pmax - main_lo + 1);
     const float r1 = a.r1[head], r2 = a.r2[head];
     float m = -INFINITY, l = 0.f, acc[16];
 #pragma unroll
@@ -619,14 +692,14 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
     const size_t esz = KVT == KV_F32 ? 4 : 2;
     const int nsplit = (int)gridDim.z;     // the visible keys' tiles are dealt round-robin to nsplit blocks (few queries, many keys)
     __syncthreads();                       // qs written (a split may have no tile at all)
-    for (long long v0 = (long long)blockIdx.z * KT; v0 < total; v0 += (long long)KT * nsplit) {
+    for (int v0 = (int)blockIdx.z * KT; v0 < total; v0 += KT * nsplit) {
         __syncthreads();                   // previous tile fully consumed
         for (int rr = 0; rr < KT / 16; ++rr) {
             const int sl = qr + 16 * rr;
-            const long long v = v0 + sl;
+            const int v = v0 + sl;
             if (v < total) {
-                const long long j = v < sink_hi ? v : main_lo + (v - sink_hi);
-                const int pg = a.bt[sg.bt_off + (int)(j / a.page)];
+                const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
+                const int pg = a.bt[sg.bt_off + j / a.page];
                 const char* src = (const char*)a.kpool + ((((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * d) * esz;
                 if (KVT != KV_F32 && (d & 7) == 0) {             // 16 bytes = 8 cached keys per lane and load
                     for (int i = ln * 8; i < d; i += 128) {
@@ -646,20 +719,14 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         float sc[KT / 16];
         float tmax = -INFINITY;
 #pragma unroll
-        for (int c = 0; c < KT / 16; ++c) sc[c] = 0.f;
-        for (int i = 0; i < d; ++i) {          // one read of q per KT / 16 keys
-            const float qv = qs[qr * d + i];
-#pragma unroll
-            for (int c = 0; c < KT / 16; ++c) sc[c] = fmaf(qv, ks[(ln + 16 * c) * ldk + i], sc[c]);
-        }
-#pragma unroll
         for (int c = 0; c < KT / 16; ++c) {
             const int sl = ln + 16 * c;
-            const long long v = v0 + sl;
-            const long long j = v < sink_hi ? v : main_lo + (v - sink_hi);
-            const float dot = sc[c];
-            const long long dist = pos - j;
-            const bool vis = qvalid && v < total && dist >= 0 && (dist < a.win || j < a.keep);
+            const int v = v0 + sl;
+            const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
+            float dot = 0.f;
+            for (int i = 0; i < d; ++i) dot = fmaf(qs[qr * d + i], ks[sl * ldk + i], dot);
+            const int dist = pos - j;
+            const bool vis = qvalid && v < total && dist >= 0 && (dist < win || j < keep);
             sc[c] = vis ? dot * a.scale - r1 * log1pf(r2 * (float)dist) : -INFINITY;
             tmax = fmaxf(tmax, sc[c]);
         }
@@ -677,15 +744,14 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         l = l * corr + psum;
         m = mn;
         __syncthreads();
-        const int kn = (int)min((long long)KT, total - v0);
+        const int kn = min(KT, total - v0);
 #pragma unroll
-        for (int c = 0; c < 16; ++c) acc[c] *= corr;
-        for (int sl = 0; sl < kn; ++sl) {      // one read of the weight per d / 16 value elements
-            const float p = ps[qr * KT + sl];
-#pragma unroll
-            for (int c = 0; c < 16; ++c) {
-                const int i = ln + 16 * c;
-                if (i < d) acc[c] = fmaf(p, ks[sl * ldk + i], acc[c]);
+        for (int c = 0; c < 16; ++c) {
+            const int i = ln + 16 * c;
+            if (i < d) {
+                float o = acc[c] * corr;
+                for (int sl = 0; sl < kn; ++sl) o = fmaf(ps[qr * KT + sl], ks[sl * ldk + i], o);
+                acc[c] = o;
             }
         }
     }
@@ -708,38 +774,29 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         if (i < d) a.out[(size_t)row * a.ldo + head * d + i] = acc[c] * inv;
     }
 }
-// merge of the splits of a tile: out = sum_z acc_z e^(m_z - M) / sum_z l_z e^(m_z - M) * gate
+// merge of the splits of a tile: out = sum_z acc_z e^(m_z - M) / sum_z l_z e^(m_z - M) * gate; one thread per (query row, element)
 __global__ __launch_bounds__(256) void lay_attn_merge_kernel(LAttnArgs a, int nsplit) {
     const int2 tile = a.tiles[blockIdx.x];
     const LaySegDev sg = a.segs[tile.x];
     const int g = blockIdx.y, nrep = a.H / a.G, d = a.d;
     const int q0 = tile.y, nq = min(LA_BQ, sg.n * nrep - q0);
-    const int qr = threadIdx.x >> 4, ln = threadIdx.x & 15;
-    if (qr >= nq) return;
-    const int qi = q0 + qr, lp = qi / nrep, head = g * nrep + (qi - lp * nrep), row = sg.row0 + lp;
-    const size_t p0 = (((size_t)blockIdx.x * a.G + g) * nsplit) * LA_BQ + qr;
-    float M = -INFINITY;
-    for (int z = 0; z < nsplit; ++z) M = fmaxf(M, a.part_ml[(p0 + (size_t)z * LA_BQ) * 2]);
-    float L = 0.f, acc[16];
-#pragma unroll
-    for (int c = 0; c < 16; ++c) acc[c] = 0.f;
-    for (int z = 0; z < nsplit; ++z) {
-        const size_t pr = p0 + (size_t)z * LA_BQ;
-        const float mz = a.part_ml[pr * 2];
-        if (mz == -INFINITY) continue;
-        const float w = expf(mz - M);
-        L = fmaf(a.part_ml[pr * 2 + 1], w, L);
-#pragma unroll
-        for (int c = 0; c < 16; ++c) {
-            const int i = ln + 16 * c;
-            if (i < d) acc[c] = fmaf(a.part_o[pr * d + i], w, acc[c]);
+    const size_t t0 = ((size_t)blockIdx.x * a.G + g) * nsplit * LA_BQ;
+    for (int idx = threadIdx.x; idx < nq * d; idx += 256) {
+        const int qr = idx / d, i = idx - qr * d;
+        const int qi = q0 + qr, lp = qi / nrep, head = g * nrep + (qi - lp * nrep), row = sg.row0 + lp;
+        float M = -INFINITY;
+#pragma unroll 8
+        for (int z = 0; z < nsplit; ++z) M = fmaxf(M, a.part_ml[(t0 + (size_t)z * LA_BQ + qr) * 2]);
+        float L = 0.f, acc = 0.f;
+#pragma unroll 8
+        for (int z = 0; z < nsplit; ++z) {
+            const size_t pr = t0 + (size_t)z * LA_BQ + qr;
+            const float mz = a.part_ml[pr * 2];
+            const float w = mz == -INFINITY ? 0.f : expf(mz - M);
+            L = fmaf(a.part_ml[pr * 2 + 1], w, L);
+            acc = fmaf(a.part_o[pr * d + i], w, acc);
         }
-    }
-    const float inv = a.proj[(size_t)row * a.ldp + a.g_off + head] / L;
-#pragma unroll
-    for (int c = 0; c < 16; ++c) {
-        const int i = ln + 16 * c;
-        if (i < d) a.out[(size_t)row * a.ldo + head * d + i] = acc[c] * inv;
+        a.out[(size_t)row * a.ldo + head * d + i] = acc * a.proj[(size_t)row * a.ldp + a.g_off + head] / L;
     }
 }
 void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s) {
