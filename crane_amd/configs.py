@@ -142,7 +142,7 @@ CONFIGS.update({
 # ---- layer-list decoders (config "architecture" + "layers"): Korupel -------------------------------------------------------
 def korupel_config(vocab: int, width: int, pattern: str, heads: int, kv_heads: int, dim: int, window: int, keep_first: int,
                    lin_heads: int, lin_dim: int, lin_vdim: int, ff: int, experts: int = 0, top: int = 0, expert_ff: int = 0,
-                   taps: int = 4, residual_mult: float = 0.3, eps: float = 1e-6) -> dict:
+                   taps: int = 4, residual_mult: float = 0.5, eps: float = 1e-5) -> dict:
     """pattern: one letter per layer -- 'a' window attention, 'l' lightning attention; upper case: mixture of experts, lower
     case: dense feed-forward.  Lightning head h of H decays with 1 - 2^-(1 + 8 h / (H - 1)): from fast to slow."""
     layers = []

@@ -44,7 +44,7 @@ def small_config():
                    layer("lightning", moe(experts=5, top=2, ff=24), **light(heads=3, dim=8, vdim=24, decay=(0.5, 0.9, 0.995))),
                    layer("lightning", DENSE, **light(heads=2, dim=24, vdim=8, decay=(0.8, 0.99))),
                    layer("attention", moe(experts=3, top=3, ff=16), **attn(heads=3, kv_heads=3, dim=24, size=33, keep_first=0, scale=0.3))],
-                  vocab=83, width=56, taps=4, mult=0.3)
+                  vocab=83, width=56, taps=5, mult=0.25, eps=2e-6)
 
 
 def random_weights(cfg, seed=0):

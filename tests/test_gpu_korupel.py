@@ -355,10 +355,12 @@ def test_synthetic_registry_model_generates(tmp_path):
 
 
 def test_bfloat16_products_on_the_shared_gemm_and_on_the_row_kernel_agree(tmp_path):
-    """Registry widths that fit the matrix-core GEMM of the other families (output widths of 128): a 100-token prompt (shared GEMM
+    """Widths that fit the matrix-core GEMM of the other families (output widths of 128 and 256): a 100-token prompt (shared GEMM
     for the products that fit), the same with the switch off (tiled kernel of this family), and token by token (row kernel)."""
     from crane_amd import configs
-    cfg = configs.get_config("tiny-korupel")
+    # dense feed-forwards only: a router's choice between two close scores may flip with the rounding of its input
+    cfg = configs.korupel_config(320, 128, "alla", heads=4, kv_heads=2, dim=32, window=24, keep_first=3, lin_heads=2, lin_dim=16,
+                                 lin_vdim=32, ff=256, taps=3, residual_mult=0.35)
     P = U.random_weights(cfg, 15)
     toks = U.tokens(100, cfg["vocab"], 15)
     want = O.forward(cfg, P, toks)
@@ -392,5 +394,26 @@ def test_decode_steps_over_hundreds_of_keys_and_a_long_portion_in_chunks(tmp_pat
         assert _err(first, want[[0, 31, 32, 33, 200, 394]]) < tol
         got = np.concatenate([m.step_batch([(s, [t], [0])])[0] for t in toks[395:]])
         assert _err(got, want[395:]) < tol
+    finally:
+        m.close()
+
+
+def test_a_step_larger_than_one_pass_is_cut_into_passes(tmp_path):
+    """Passes of 32 rows: a 100-token portion beside a 45-token one and a single token runs as five passes; the wanted rows come
+    back in the order of the items whatever pass they fell into."""
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 17)
+    reqs = [U.tokens(n, cfg["vocab"], 70 + i) for i, n in enumerate((100, 45, 9))]
+    want = [O.forward(cfg, P, t) for t in reqs]
+    m = _load(tmp_path, cfg, P, prefill_chunk=32)
+    try:
+        s = [m.seq_alloc() for _ in reqs]
+        m.step_batch([(s[2], reqs[2][:8], [])])
+        w0, w1 = [0, 31, 32, 63, 64, 99], [10, 44]
+        got, greedy = m.step_batch([(s[0], reqs[0], w0), (s[1], reqs[1], w1), (s[2], reqs[2][8:], None)])
+        ref = np.concatenate([want[0][w0], want[1][w1], want[2][8:9]])
+        assert got.shape == ref.shape and _err(got, ref) < TOL_F32
+        assert list(greedy) == [int(np.argmax(r)) for r in got]
+        assert [m.seq_len(x) for x in s] == [100, 45, 9]
     finally:
         m.close()
