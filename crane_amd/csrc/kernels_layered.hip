@@ -774,6 +774,150 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         if (i < d) a.out[(size_t)row * a.ldo + head * d + i] = acc[c] * inv;
     }
 }
+// Matrix-core form for prompt passes in the bfloat16 format (head size a multiple of 16, up to 128): 64 query rows per block, one
+// wave per 16 of them, 64-key tiles.  S = Q K^T from the bf16-rounded q and the cached bf16 keys (exact products, f32 sums);
+// mask, distance penalty, running max / sum and the weights stay f32 as in lay_attn_kernel; the weights enter P V (V = K) as a
+// bf16 hi + lo pair, two products per tile, so that they keep 16 significand bits; exp and log are the hardware's (v_exp_f32 /
+// v_log_f32, about 1e-6 relative: the format's own rounding is three orders above that).  Fragment layout of v_mfma_f32_16x16x16_bf16:
+// A[i = lane % 16][k = 4 (lane / 16) ..], B[k = 4 (lane / 16) ..][j = lane % 16], D[i = 4 (lane / 16) + r][j = lane % 16].
+constexpr int LM_BQ = 64, LM_KT = 64;
+__global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    const int d = a.d, ldq = d + 8, ldp = LM_KT + 8;
+    uint16_t* Qs = smem;                              // [64][d + 8]
+    uint16_t* Ks = Qs + LM_BQ * ldq;                  // [64][d + 8]
+    uint16_t* Ph = Ks + LM_KT * ldq;                  // [4 waves][16][72] hi
+    uint16_t* Pl = Ph + 4 * 16 * ldp;                 // ... lo
+    const int2 tile = a.tiles[blockIdx.x];
+    const LaySegDev sg = a.segs[tile.x];
+    const int g = blockIdx.y, nrep = a.H / a.G;
+    const int q0 = tile.y, nq = min(LM_BQ, sg.n * nrep - q0);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 15, lg = lane >> 4;
+    const int win = (int)min(a.win, 1ll << 30), keep = (int)min(a.keep, 1ll << 30);
+    // q rows -> bf16
+    for (int idx = tid; idx < LM_BQ * (d / 4); idx += 256) {
+        const int qr = idx / (d / 4), i = (idx - qr * (d / 4)) * 4;
+        u32x2 pk = {0u, 0u};
+        if (qr < nq) {
+            const int qi = q0 + qr, lp = qi / nrep, head = g * nrep + (qi - lp * nrep);
+            const float* src = a.proj + (size_t)(sg.row0 + lp) * a.ldp + a.q_off + head * d + i;
+            pk.x = pack_bf16x2(src[0], src[1]); pk.y = pack_bf16x2(src[2], src[3]);
+        }
+        *(u32x2*)&Qs[qr * ldq + i] = pk;
+    }
+    // this lane's four query rows (accumulator rows 4 lg + r of the wave's 16)
+    int qpos[4], qhead[4], qrow[4]; bool qok[4]; float r1[4], r2[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int qr = wave * 16 + 4 * lg + r;
+        qok[r] = qr < nq;
+        const int qi = q0 + (qok[r] ? qr : 0), lp = qi / nrep;
+        qhead[r] = g * nrep + (qi - lp * nrep);
+        qpos[r] = sg.start_pos + lp;
+        qrow[r] = sg.row0 + lp;
+        r1[r] = a.r1[qhead[r]]; r2[r] = a.r2[qhead[r]];
+    }
+    const int pmin = sg.start_pos + q0 / nrep, pmax = sg.start_pos + (q0 + nq - 1) / nrep;
+    const int main_lo = max(0, pmin - win + 1);
+    const int sink_hi = min(keep, main_lo);
+    const int total = sink_hi + (pmax - main_lo + 1);
+    f32x4 O[8];
+#pragma unroll
+    for (int n = 0; n < 8; ++n) O[n] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
+    const int nd = d / 16;
+    uint16_t* ph = Ph + wave * 16 * ldp;
+    uint16_t* pl = Pl + wave * 16 * ldp;
+    for (int v0 = 0; v0 < total; v0 += LM_KT) {
+        __syncthreads();                   // previous tile consumed (first round: Qs written)
+        for (int idx = tid; idx < LM_KT * (d / 8); idx += 256) {
+            const int sl = idx / (d / 8), i = (idx - sl * (d / 8)) * 8;
+            const int v = v0 + sl;
+            u32x4 pk = {0u, 0u, 0u, 0u};
+            if (v < total) {
+                const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
+                const int pg = a.bt[sg.bt_off + j / a.page];
+                pk = *(const u32x4*)((const uint16_t*)a.kpool + (((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * d + i);
+            }
+            *(u32x4*)&Ks[sl * ldq + i] = pk;
+        }
+        __syncthreads();
+        f32x4 S[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int kk = 0; kk < nd; ++kk) {
+            const bf16x4 qa = *(const bf16x4*)&Qs[(wave * 16 + lr) * ldq + kk * 16 + 4 * lg];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const bf16x4 kb = *(const bf16x4*)&Ks[(t * 16 + lr) * ldq + kk * 16 + 4 * lg];
+                S[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(qa, kb, S[t], 0, 0, 0);
+            }
+        }
+        float corr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float sc[4], tmax = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int v = v0 + t * 16 + lr;
+                const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
+                const int dist = qpos[r] - j;
+                const bool vis = qok[r] && v < total && dist >= 0 && (dist < win || j < keep);
+                sc[t] = vis ? S[t][r] * a.scale - r1[r] * __logf(1.f + r2[r] * (float)dist) : -INFINITY;
+                tmax = fmaxf(tmax, sc[t]);
+            }
+            tmax = row16_max(tmax);
+            const float mn = fmaxf(m[r], tmax);
+            corr[r] = mn == -INFINITY ? 1.f : __expf(m[r] - mn);
+            float psum = 0.f;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float p = sc[t] == -INFINITY ? 0.f : __expf(sc[t] - mn);
+                psum += p;
+                const uint16_t hi = f32_to_bf16(p);
+                ph[(4 * lg + r) * ldp + t * 16 + lr] = hi;
+                pl[(4 * lg + r) * ldp + t * 16 + lr] = f32_to_bf16(p - bf16_to_f32(hi));
+            }
+            psum = row16_sum(psum);
+            l[r] = l[r] * corr[r] + psum;
+            m[r] = mn;
+        }
+#pragma unroll
+        for (int n = 0; n < 8; ++n)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) O[n][r] *= corr[r];
+        __syncthreads();                   // the wave's weights are in LDS
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const bf16x4 ah = *(const bf16x4*)&ph[lr * ldp + ks * 16 + 4 * lg];
+            const bf16x4 al = *(const bf16x4*)&pl[lr * ldp + ks * 16 + 4 * lg];
+#pragma unroll
+            for (int n = 0; n < 8; ++n) {
+                if (n < nd) {
+                    bf16x4 vb;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) vb[e] = (short)Ks[(ks * 16 + 4 * lg + e) * ldq + n * 16 + lr];
+                    O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah, vb, O[n], 0, 0, 0);
+                    O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(al, vb, O[n], 0, 0, 0);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (!qok[r]) continue;
+        const float inv = a.proj[(size_t)qrow[r] * a.ldp + a.g_off + qhead[r]] / l[r];
+#pragma unroll
+        for (int n = 0; n < 8; ++n)
+            if (n < nd) a.out[(size_t)qrow[r] * a.ldo + qhead[r] * d + n * 16 + lr] = O[n][r] * inv;
+    }
+}
+void launch_lay_attn_mfma(const LAttnArgs& a, hipStream_t s) {
+    if (a.ntiles <= 0) return;
+    const size_t lds = ((size_t)(LM_BQ + LM_KT) * (a.d + 8) + 2 * 4 * 16 * (LM_KT + 8)) * sizeof(uint16_t);
+    hipLaunchKernelGGL(lay_attn_mfma_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(256), lds, s, a);
+}
+
 // merge of the splits of a tile: out = sum_z acc_z e^(m_z - M) / sum_z l_z e^(m_z - M) * gate; one thread per (query row, element)
 __global__ __launch_bounds__(256) void lay_attn_merge_kernel(LAttnArgs a, int nsplit) {
     const int2 tile = a.tiles[blockIdx.x];

@@ -39,6 +39,7 @@ struct Layered {
     // bfloat16 format, products of 32 rows or more whose shape fits (N % 128 == 0, K % 32 == 0): the matrix-core GEMM the other
     // families' prompt passes use (kernels_prefill.hip / kernels_gemm256.hip), plain bf16 activations; cm_debug_set("lay_shared_gemm", 0): never
     bool shared_gemm = true;
+    bool attn_mfma = true;             // bfloat16 format, prompt passes: the matrix-core attention (cm_debug_set("lay_attn_mfma", 0): never)
     uint16_t* Abf = nullptr;           // [cap rounded up to 256][widest K] bf16 A operand
     float *G1 = nullptr, *G2 = nullptr;   // [cap][widest dense ff] the two products of a gated feed-forward
     float* U = nullptr;                // lightning attention, chunk-parallel form: [chunks of a pass][widest H d e] f32
@@ -413,7 +414,7 @@ void Model::alloc_runtime_layered() {
     CM_HIP(hipHostMalloc((void**)&L.h_greedy, Layered::LOGIT_ROWS * sizeof(uint32_t)));
     // one table upload per pass: ids | rowseg | wanted rows | segments | page tables | attention tiles per group size
     size_t tiles = 0;
-    for (int nrep : L.nreps) tiles += 2 * (cap * (size_t)nrep / 16 + (size_t)MAXB + 1);
+    for (int nrep : L.nreps) tiles += 2 * (cap * (size_t)nrep / 16 + (size_t)MAXB + 1) + 2 * (cap * (size_t)nrep / LAY_ATTN_MFMA_ROWS + (size_t)MAXB + 1);
     tiles += 2 * (cap / LAY_LIGHT_CHUNK + (size_t)MAXB + 1);      // lightning chunks
     L.tab_ints = 3 * cap + (size_t)MAXB * (sizeof(LaySegDev) / 4) + (size_t)MAXB * max_pages_per_seq + tiles + 64;
     L.d_tab = dalloc<int32_t>(L.tab_ints);
@@ -430,6 +431,10 @@ size_t Model::layered_capture(float* out, size_t n) const {
 void Model::layered_set_shared_gemm(bool on) {
     if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
     lay->shared_gemm = on;
+}
+void Model::layered_set_attn_mfma(bool on) {
+    if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
+    lay->attn_mfma = on;
 }
 void Model::layered_set_capture(bool on) {
     if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
@@ -528,13 +533,18 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             row += n;
             q.len += n;                        // the cache holds these positions once the pass has run
         }
-        std::map<int, std::pair<size_t, int>> tiles;      // nrep -> (offset, count)
+        std::map<int, std::pair<size_t, int>> tiles, tiles64;      // nrep -> (offset, count): 16 / 64 query rows per tile
         for (int nrep : L.nreps) {
             if (o & 1) ++o;                    // int2 entries
             const size_t o_t = o; int cnt = 0;
             for (int k = 0; k < nseg; ++k)
                 for (int q0 = 0; q0 < t_segs[k].n * nrep; q0 += 16) { tab[o++] = k; tab[o++] = q0; ++cnt; }
             tiles[nrep] = {o_t, cnt};
+            const size_t o_m = o; cnt = 0;
+            if (!all_decode)
+                for (int k = 0; k < nseg; ++k)
+                    for (int q0 = 0; q0 < t_segs[k].n * nrep; q0 += LAY_ATTN_MFMA_ROWS) { tab[o++] = k; tab[o++] = q0; ++cnt; }
+            tiles64[nrep] = {o_m, cnt};
         }
         if (o & 1) ++o;
         const size_t o_chunks = o;
@@ -606,6 +616,11 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     a.nsplit = std::max(1, std::min({32, key_tiles, 256 / blocks, Layered::ATT_PARTS / blocks}));
                     a.part_o = L.att_po; a.part_ml = L.att_pml;
                 }
+                if (L.attn_mfma && kv_mode == KV_BF16 && !all_decode && max_n >= 16 && sp.dim % 16 == 0 && sp.dim <= 128) {
+                    const auto& tm = tiles64[sp.heads / sp.kv_heads];
+                    a.tiles = (const int2*)(L.d_tab + tm.first); a.ntiles = tm.second;
+                    launch_lay_attn_mfma(a, s);
+                } else
                 launch_lay_attn(a, kv_mode, s);
                 on = sp.heads * sp.dim; oa = L.O;
             } else {
