@@ -784,8 +784,9 @@ constexpr int LM_BQ = 64, LM_KT = 64;
 __global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
     const int d = a.d, ldq = d + 8, ldp = LM_KT + 8;
-    uint16_t* Qs = smem;                              // [64][d + 8]
-    uint16_t* Ks = Qs + LM_BQ * ldq;                  // [64][d + 8]
+    uint16_t* Qs = smem;                              // [64][d + 8] until the q fragments sit in registers, then:
+    uint16_t* Kt = smem;                              // [d][72] the key tile transposed (the B operand of P V: 4 keys of one element)
+    uint16_t* Ks = smem + max(LM_BQ * ldq, d * ldp);  // [64][d + 8]
     uint16_t* Ph = Ks + LM_KT * ldq;                  // [4 waves][16][72] hi
     uint16_t* Pl = Ph + 4 * 16 * ldp;                 // ... lo
     const int2 tile = a.tiles[blockIdx.x];
@@ -828,8 +829,13 @@ __global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
     const int nd = d / 16;
     uint16_t* ph = Ph + wave * 16 * ldp;
     uint16_t* pl = Pl + wave * 16 * ldp;
+    __syncthreads();                       // Qs written
+    bf16x4 qf[8];
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk)
+        qf[kk] = kk < nd ? *(const bf16x4*)&Qs[(wave * 16 + lr) * ldq + kk * 16 + 4 * lg] : (bf16x4){0, 0, 0, 0};
     for (int v0 = 0; v0 < total; v0 += LM_KT) {
-        __syncthreads();                   // previous tile consumed (first round: Qs written)
+        __syncthreads();                   // previous tile consumed (first round: q fragments read, Qs free for Kt)
         for (int idx = tid; idx < LM_KT * (d / 8); idx += 256) {
             const int sl = idx / (d / 8), i = (idx - sl * (d / 8)) * 8;
             const int v = v0 + sl;
@@ -840,13 +846,19 @@ __global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
                 pk = *(const u32x4*)((const uint16_t*)a.kpool + (((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * d + i);
             }
             *(u32x4*)&Ks[sl * ldq + i] = pk;
+            Kt[(i + 0) * ldp + sl] = (uint16_t)(pk.x & 0xFFFFu); Kt[(i + 1) * ldp + sl] = (uint16_t)(pk.x >> 16);
+            Kt[(i + 2) * ldp + sl] = (uint16_t)(pk.y & 0xFFFFu); Kt[(i + 3) * ldp + sl] = (uint16_t)(pk.y >> 16);
+            Kt[(i + 4) * ldp + sl] = (uint16_t)(pk.z & 0xFFFFu); Kt[(i + 5) * ldp + sl] = (uint16_t)(pk.z >> 16);
+            Kt[(i + 6) * ldp + sl] = (uint16_t)(pk.w & 0xFFFFu); Kt[(i + 7) * ldp + sl] = (uint16_t)(pk.w >> 16);
         }
         __syncthreads();
         f32x4 S[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        for (int kk = 0; kk < nd; ++kk) {
-            const bf16x4 qa = *(const bf16x4*)&Qs[(wave * 16 + lr) * ldq + kk * 16 + 4 * lg];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            if (kk >= nd) break;
+            const bf16x4 qa = qf[kk];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const bf16x4 kb = *(const bf16x4*)&Ks[(t * 16 + lr) * ldq + kk * 16 + 4 * lg];
@@ -894,9 +906,7 @@ __global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
 #pragma unroll
             for (int n = 0; n < 8; ++n) {
                 if (n < nd) {
-                    bf16x4 vb;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) vb[e] = (short)Ks[(ks * 16 + 4 * lg + e) * ldq + n * 16 + lr];
+                    const bf16x4 vb = *(const bf16x4*)&Kt[(n * 16 + lr) * ldp + ks * 16 + 4 * lg];
                     O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah, vb, O[n], 0, 0, 0);
                     O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(al, vb, O[n], 0, 0, 0);
                 }
@@ -914,7 +924,7 @@ __global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
 }
 void launch_lay_attn_mfma(const LAttnArgs& a, hipStream_t s) {
     if (a.ntiles <= 0) return;
-    const size_t lds = ((size_t)(LM_BQ + LM_KT) * (a.d + 8) + 2 * 4 * 16 * (LM_KT + 8)) * sizeof(uint16_t);
+    const size_t lds = ((size_t)std::max(LM_BQ * (a.d + 8), a.d * (LM_KT + 8)) + (size_t)LM_KT * (a.d + 8) + 2 * 4 * 16 * (LM_KT + 8)) * sizeof(uint16_t);
     hipLaunchKernelGGL(lay_attn_mfma_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(256), lds, s, a);
 }
 
