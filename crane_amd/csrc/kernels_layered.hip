@@ -774,21 +774,21 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         if (i < d) a.out[(size_t)row * a.ldo + head * d + i] = acc[c] * inv;
     }
 }
-// Matrix-core form for prompt passes in the bfloat16 format (head size a multiple of 16, up to 128): 64 query rows per block, one
-// wave per 16 of them, 64-key tiles.  S = Q K^T from the bf16-rounded q and the cached bf16 keys (exact products, f32 sums);
+// Matrix-core form for prompt passes in the bfloat16 format (head size a multiple of 16, up to 128): LAY_ATTN_MFMA_ROWS query rows per
+// block, one wave per 16 of them, 64-key tiles (32-row blocks, two or three resident per CU, measured slower: 474 against 423 us for 2048 tokens).  S = Q K^T from the bf16-rounded q and the cached bf16 keys (exact products, f32 sums);
 // mask, distance penalty, running max / sum and the weights stay f32 as in lay_attn_kernel; the weights enter P V (V = K) as a
 // bf16 hi + lo pair, two products per tile, so that they keep 16 significand bits; exp and log are the hardware's (v_exp_f32 /
 // v_log_f32, about 1e-6 relative: the format's own rounding is three orders above that).  Fragment layout of v_mfma_f32_16x16x16_bf16:
 // A[i = lane % 16][k = 4 (lane / 16) ..], B[k = 4 (lane / 16) ..][j = lane % 16], D[i = 4 (lane / 16) + r][j = lane % 16].
-constexpr int LM_BQ = 64, LM_KT = 64;
-__global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
+constexpr int LM_BQ = LAY_ATTN_MFMA_ROWS, LM_KT = 64, LM_NT = LM_BQ * 4, LM_NW = LM_BQ / 16;    // threads, waves
+__global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
     const int d = a.d, ldq = d + 8, ldp = LM_KT + 8;
-    uint16_t* Qs = smem;                              // [64][d + 8] until the q fragments sit in registers, then:
+    uint16_t* Qs = smem;                              // [rows][d + 8] until the q fragments sit in registers, then:
     uint16_t* Kt = smem;                              // [d][72] the key tile transposed (the B operand of P V: 4 keys of one element)
     uint16_t* Ks = smem + max(LM_BQ * ldq, d * ldp);  // [64][d + 8]
-    uint16_t* Ph = Ks + LM_KT * ldq;                  // [4 waves][16][72] hi
-    uint16_t* Pl = Ph + 4 * 16 * ldp;                 // ... lo
+    uint16_t* Ph = Ks + LM_KT * ldq;                  // [waves][16][72] hi
+    uint16_t* Pl = Ph + LM_NW * 16 * ldp;                 // ... lo
     const int2 tile = a.tiles[blockIdx.x];
     const LaySegDev sg = a.segs[tile.x];
     const int g = blockIdx.y, nrep = a.H / a.G;
@@ -796,7 +796,7 @@ __global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 15, lg = lane >> 4;
     const int win = (int)min(a.win, 1ll << 30), keep = (int)min(a.keep, 1ll << 30);
     // q rows -> bf16
-    for (int idx = tid; idx < LM_BQ * (d / 4); idx += 256) {
+    for (int idx = tid; idx < LM_BQ * (d / 4); idx += LM_NT) {
         const int qr = idx / (d / 4), i = (idx - qr * (d / 4)) * 4;
         u32x2 pk = {0u, 0u};
         if (qr < nq) {
@@ -836,7 +836,7 @@ __global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
         qf[kk] = kk < nd ? *(const bf16x4*)&Qs[(wave * 16 + lr) * ldq + kk * 16 + 4 * lg] : (bf16x4){0, 0, 0, 0};
     for (int v0 = 0; v0 < total; v0 += LM_KT) {
         __syncthreads();                   // previous tile consumed (first round: q fragments read, Qs free for Kt)
-        for (int idx = tid; idx < LM_KT * (d / 8); idx += 256) {
+        for (int idx = tid; idx < LM_KT * (d / 8); idx += LM_NT) {
             const int sl = idx / (d / 8), i = (idx - sl * (d / 8)) * 8;
             const int v = v0 + sl;
             u32x4 pk = {0u, 0u, 0u, 0u};
@@ -924,8 +924,8 @@ __global__ __launch_bounds__(256) void lay_attn_mfma_kernel(LAttnArgs a) {
 }
 void launch_lay_attn_mfma(const LAttnArgs& a, hipStream_t s) {
     if (a.ntiles <= 0) return;
-    const size_t lds = ((size_t)std::max(LM_BQ * (a.d + 8), a.d * (LM_KT + 8)) + (size_t)LM_KT * (a.d + 8) + 2 * 4 * 16 * (LM_KT + 8)) * sizeof(uint16_t);
-    hipLaunchKernelGGL(lay_attn_mfma_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(256), lds, s, a);
+    const size_t lds = ((size_t)std::max(LM_BQ * (a.d + 8), a.d * (LM_KT + 8)) + (size_t)LM_KT * (a.d + 8) + 2 * LM_NW * 16 * (LM_KT + 8)) * sizeof(uint16_t);
+    hipLaunchKernelGGL(lay_attn_mfma_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(LM_NT), lds, s, a);
 }
 
 // merge of the splits of a tile: out = sum_z acc_z e^(m_z - M) / sum_z l_z e^(m_z - M) * gate; one thread per (query row, element)

@@ -104,7 +104,8 @@ struct LAttnArgs {
 void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int kvt, const int32_t* bt, const LaySegDev* segs,
                          const int32_t* rowseg, int T, int G, int d, int page, hipStream_t s);
 void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s);    // kvt: KV_BF16 | KV_F32
-// bf16 key pages, d % 16 == 0, d <= 128: the matrix-core form; a.tiles lists {segment, first query row} in steps of 64 rows
+// bf16 key pages, d % 16 == 0, d <= 128: the matrix-core form; a.tiles lists {segment, first query row} in steps of
+// LAY_ATTN_MFMA_ROWS rows, longest key range first
 constexpr int LAY_ATTN_MFMA_ROWS = 64;
 void launch_lay_attn_mfma(const LAttnArgs& a, hipStream_t s);
 

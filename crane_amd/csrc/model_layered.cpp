@@ -541,9 +541,14 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 for (int q0 = 0; q0 < t_segs[k].n * nrep; q0 += 16) { tab[o++] = k; tab[o++] = q0; ++cnt; }
             tiles[nrep] = {o_t, cnt};
             const size_t o_m = o; cnt = 0;
-            if (!all_decode)
+            if (!all_decode) {
                 for (int k = 0; k < nseg; ++k)
                     for (int q0 = 0; q0 < t_segs[k].n * nrep; q0 += LAY_ATTN_MFMA_ROWS) { tab[o++] = k; tab[o++] = q0; ++cnt; }
+                // blocks with the longest key range first: the short ones fill the tail of the launch
+                int2* tl = (int2*)(tab + o_m);
+                std::stable_sort(tl, tl + cnt, [&](const int2& x, const int2& y) {
+                    return t_segs[x.x].start_pos + x.y / nrep > t_segs[y.x].start_pos + y.y / nrep; });
+            }
             tiles64[nrep] = {o_m, cnt};
         }
         if (o & 1) ++o;
