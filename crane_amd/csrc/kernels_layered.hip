@@ -11,8 +11,10 @@ namespace cm {
 
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-__device__ __forceinline__ float lay_act(float v, int act) {
+__device__ __forceinline__ float lay_act(float v, int act, float param = 1.f) {
     switch (act) {
+        case LACT_RELU2: { const float r = fmaxf(v, 0.f); return r * r; }
+        case LACT_LOGSIG: return param * (fminf(v, 0.f) - log1pf(expf(-fabsf(v))));      // ln sigmoid(v), no overflow either way
         case LACT_SILU: return v / (1.f + __expf(-v));
         case LACT_SIGMOID: return 1.f / (1.f + __expf(-v));
         case LACT_GELU_TANH: {
@@ -65,6 +67,121 @@ void launch_lay_rms_rows(const float* x, const int32_t* rows, const float* w, fl
     hipLaunchKernelGGL(lay_rms_rows_kernel, dim3((unsigned)n_rows), dim3(256), 0, s, x, rows, w, out, W, eps);
 }
 
+__global__ __launch_bounds__(256) void lay_rms_rows2_kernel(const float* __restrict__ x, const float* __restrict__ w1,
+                                                            const float* __restrict__ w2, float* __restrict__ out1, float* __restrict__ out2,
+                                                            int W, float eps) {
+    __shared__ float red[4];
+    const float* xr = x + (size_t)blockIdx.x * W;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) { const float v = xr[c]; ss += v * v; }
+    ss = block_sum(ss, red);
+    const float rs = 1.f / sqrtf(ss / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float v = xr[c] * rs;
+        out1[(size_t)blockIdx.x * W + c] = v * w1[c];
+        if (out2) out2[(size_t)blockIdx.x * W + c] = v * w2[c];
+    }
+}
+void launch_lay_rms_rows2(const float* x, const float* w1, const float* w2, float* out1, float* out2, int T, int W, float eps, hipStream_t s) {
+    if (T <= 0) return;
+    hipLaunchKernelGGL(lay_rms_rows2_kernel, dim3((unsigned)T), dim3(256), 0, s, x, w1, w2, out1, out2, W, eps);
+}
+
+__global__ __launch_bounds__(256) void lay_rms_cols_kernel(const float* src, int lds, int off, int n, const float* __restrict__ w, float* dst,
+                                                           int ldd, float eps) {
+    __shared__ float red[4];
+    const float* xr = src + (size_t)blockIdx.x * lds + off;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < n; c += 256) { const float v = xr[c]; ss += v * v; }
+    ss = block_sum(ss, red);           // every read of the row is done behind this barrier: dst may be the same memory
+    const float rs = 1.f / sqrtf(ss / (float)n + eps);
+    for (int c = threadIdx.x; c < n; c += 256) dst[(size_t)blockIdx.x * ldd + c] = xr[c] * rs * w[c];
+}
+void launch_lay_rms_cols(const float* src, int lds, int off, int n, const float* w, float* dst, int ldd, int T, float eps, hipStream_t s) {
+    if (T <= 0 || n <= 0) return;
+    hipLaunchKernelGGL(lay_rms_cols_kernel, dim3((unsigned)T), dim3(256), 0, s, src, lds, off, n, w, dst, ldd, eps);
+}
+
+__global__ __launch_bounds__(256) void lay_add_rows_kernel(float* __restrict__ x, const float* __restrict__ y1, const float* __restrict__ y2,
+                                                           size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) x[i] += y2 ? y1[i] + y2[i] : y1[i];
+}
+void launch_lay_add_rows(float* x, const float* y1, const float* y2, size_t n, hipStream_t s) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(lay_add_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, y1, y2, n);
+}
+
+__global__ __launch_bounds__(256) void lay_add_norm2_shift_decode_kernel(float* __restrict__ x, const float* __restrict__ y1,
+                                                                         const float* __restrict__ y2, const float* __restrict__ w1,
+                                                                         const float* __restrict__ w2, float eps, float* __restrict__ out1,
+                                                                         float* __restrict__ out2, const float* __restrict__ cw,
+                                                                         float* __restrict__ conv_pool, size_t slot_stride, size_t off,
+                                                                         const LaySegDev* __restrict__ segs, int W) {
+    __shared__ float red[4];
+    const LaySegDev sg = segs[blockIdx.x];
+    const size_t r = (size_t)sg.row0 * W;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float v = x[r + c];
+        if (y1) { v += y2 ? y1[r + c] + y2[r + c] : y1[r + c]; x[r + c] = v; }     // read back below by the same thread
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float rs = 1.f / sqrtf(ss / (float)W + eps);
+    float* prev = conv_pool + (size_t)sg.slot * slot_stride + off;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float v = x[r + c] * rs;
+        const float h = v * w1[c];
+        float acc = h;
+        acc += cw[2 * c] * prev[c];
+        acc += cw[2 * c + 1] * h;
+        out1[r + c] = acc;
+        prev[c] = h;
+        if (out2) out2[r + c] = v * w2[c];
+    }
+}
+void launch_lay_add_norm2_shift_decode(float* x, const float* y1, const float* y2, const float* w1, const float* w2, float eps, float* out1,
+                                       float* out2, const float* cw, float* conv_pool, size_t slot_stride, size_t off, const LaySegDev* segs,
+                                       int T, int W, hipStream_t s) {
+    if (T <= 0) return;
+    hipLaunchKernelGGL(lay_add_norm2_shift_decode_kernel, dim3((unsigned)T), dim3(256), 0, s, x, y1, y2, w1, w2, eps, out1, out2, cw, conv_pool,
+                       slot_stride, off, segs, W);
+}
+
+// rotation by position: the angle and its sine / cosine are f32 (sincosf reduces the argument exactly)
+__global__ __launch_bounds__(256) void lay_rope_kernel(const float* src, int lds, int s_vstride, float* dst, int ldd, int d_vstride, int nvec,
+                                                       int len, int dims, const float* __restrict__ freq, float mag,
+                                                       const LaySegDev* __restrict__ segs, const int32_t* __restrict__ rowseg) {
+    const int r = blockIdx.x;
+    const LaySegDev sg = segs[rowseg[r]];
+    const float pos = (float)(sg.start_pos + (r - sg.row0));
+    const int hp = (len + 1) / 2;
+    for (int idx = threadIdx.x; idx < nvec * hp; idx += 256) {
+        const int v = idx / hp, i = idx - v * hp;
+        const float* sp = src + (size_t)r * lds + (size_t)v * s_vstride + 2 * i;
+        float* dp = dst + (size_t)r * ldd + (size_t)v * d_vstride + 2 * i;
+        const bool two = 2 * i + 1 < len;
+        const float a = sp[0], b = two ? sp[1] : 0.f;
+        if (2 * i + 1 < dims) {
+            float sn, cs;
+            sincosf(pos * freq[i], &sn, &cs);
+            sn *= mag; cs *= mag;
+            dp[0] = a * cs - b * sn;
+            dp[1] = b * cs + a * sn;
+        } else {
+            dp[0] = a;
+            if (two) dp[1] = b;
+        }
+    }
+}
+void launch_lay_rope(const float* src, int lds, int s_vstride, float* dst, int ldd, int d_vstride, int nvec, int len, int dims,
+                     const float* freq, float mag, const LaySegDev* segs, const int32_t* rowseg, int T, hipStream_t s) {
+    if (T <= 0 || nvec <= 0 || len <= 0) return;
+    hipLaunchKernelGGL(lay_rope_kernel, dim3((unsigned)T), dim3(256), 0, s, src, lds, s_vstride, dst, ldd, d_vstride, nvec, len, dims, freq, mag,
+                       segs, rowseg);
+}
+
 __global__ __launch_bounds__(256) void lay_rms_gate_kernel(const float* __restrict__ o, const float* __restrict__ gate, int ldg,
                                                            const float* __restrict__ w, float* __restrict__ out, int N, float eps) {
     __shared__ float red[4];
@@ -76,8 +193,31 @@ __global__ __launch_bounds__(256) void lay_rms_gate_kernel(const float* __restri
     const float rs = 1.f / sqrtf(ss / (float)N + eps);
     for (int c = threadIdx.x; c < N; c += 256) out[(size_t)r * N + c] = orow[c] * rs * w[c] * gate[(size_t)r * ldg + c];
 }
-void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s) {
+// the same with the root mean square over groups of `group` columns: one wave per group
+__global__ __launch_bounds__(256) void lay_rms_gate_group_kernel(const float* __restrict__ o, const float* __restrict__ gate, int ldg,
+                                                                 const float* __restrict__ w, float* __restrict__ out, int N, int group,
+                                                                 int shared_w, float eps) {
+    const int r = blockIdx.x, lane = threadIdx.x & 63;
+    const int ngroups = N / group;
+    for (int g = (int)blockIdx.y * 4 + (int)(threadIdx.x >> 6); g < ngroups; g += 4 * (int)gridDim.y) {
+        const float* og = o + (size_t)r * N + (size_t)g * group;
+        float ss = 0.f;
+        for (int c = lane; c < group; c += 64) { const float v = og[c]; ss += v * v; }
+        ss = wave_sum(ss);
+        const float rs = 1.f / sqrtf(ss / (float)group + eps);
+        for (int c = lane; c < group; c += 64)
+            out[(size_t)r * N + (size_t)g * group + c] = og[c] * rs * w[shared_w ? c : g * group + c] * gate[(size_t)r * ldg + (size_t)g * group + c];
+    }
+}
+void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s,
+                         int group, bool shared_w) {
     if (T <= 0) return;
+    if (group > 0 && group < N) {
+        const int ngroups = N / group;
+        hipLaunchKernelGGL(lay_rms_gate_group_kernel, dim3((unsigned)T, (unsigned)std::min(16, (ngroups + 3) / 4)), dim3(256), 0, s, o, gate, ldg, w,
+                           out, N, group, shared_w ? 1 : 0, eps);
+        return;
+    }
     hipLaunchKernelGGL(lay_rms_gate_kernel, dim3((unsigned)T), dim3(256), 0, s, o, gate, ldg, w, out, N, eps);
 }
 
@@ -329,7 +469,7 @@ void launch_lay_norm_canon_decode(const float* x, const float* nw, float eps, fl
 // ------------------------------------------------------------------------------------------------------------------
 constexpr int LG_BM = 64, LG_BN = 64;
 
-struct LgTile { int p0, rows, n0; const uint16_t* W; const uint16_t* W2; };
+struct LgTile { int p0, rows, n0; const uint16_t* W; const uint16_t* W2; const float* A; size_t coff; };
 
 __device__ __forceinline__ bool lg_tile(const LGemmArgs& a, LgTile& t) {
     const int g = blockIdx.z;
@@ -342,15 +482,18 @@ __device__ __forceinline__ bool lg_tile(const LGemmArgs& a, LgTile& t) {
     t.n0 = blockIdx.y * LG_BN;
     t.W = a.W + (size_t)g * a.w_stride;
     t.W2 = a.W2 ? a.W2 + (size_t)g * a.w_stride : nullptr;
+    t.A = a.A + (a.grp_off ? 0 : (size_t)g * a.a_goff);
+    t.coff = a.grp_off ? 0 : (size_t)g * a.c_goff;
     return true;
 }
 
-__device__ __forceinline__ void lg_store(const LGemmArgs& a, int p, int n, float v, float v2, bool dual) {
+__device__ __forceinline__ void lg_store(const LGemmArgs& a, size_t coff, int p, int n, float v, float v2, bool dual) {
     if (a.bias) v += a.bias[n];
     if (dual) v = lay_act(v, a.act) * v2;
-    else v = lay_act(v, n < a.act_split ? a.act : a.act2);
+    else v = lay_act(v, n < a.act_split ? a.act : a.act2, a.act_param);
+    if (a.mul) v *= a.mul[(size_t)p * a.ldm + coff + n];
     const size_t row = a.c_idx ? (size_t)a.c_idx[p] : (size_t)p;
-    a.C[row * a.ldc + n] = v;
+    a.C[row * a.ldc + coff + n] = v;
 }
 
 // f32 FMA form: 4 x 4 outputs per thread, k in steps of 16
@@ -376,7 +519,7 @@ __global__ __launch_bounds__(256) void lgemm_f32_kernel(LGemmArgs a) {
         for (int i = 0; i < 4; ++i) {
             const int idx = tid + i * 256, r = idx >> 4, kk = idx & 15, k = k0 + kk;
             const int ar = arow[r];
-            As[kk][r] = (ar >= 0 && k < a.K) ? a.A[(size_t)ar * a.lda + k] : 0.f;
+            As[kk][r] = (ar >= 0 && k < a.K) ? t.A[(size_t)ar * a.lda + k] : 0.f;
             const int n = t.n0 + r;
             const bool ok = n < a.N && k < a.K;
             Bs[kk][r] = ok ? bf16_to_f32(t.W[(size_t)n * a.K + k]) : 0.f;
@@ -403,7 +546,7 @@ __global__ __launch_bounds__(256) void lgemm_f32_kernel(LGemmArgs a) {
         if (r >= t.rows) continue;
         for (int j = 0; j < 4; ++j) {
             const int n = t.n0 + tx * 4 + j;
-            if (n < a.N) lg_store(a, t.p0 + r, n, acc[i][j], acc2[i][j], DUAL);
+            if (n < a.N) lg_store(a, t.coff, t.p0 + r, n, acc[i][j], acc2[i][j], DUAL);
         }
     }
 }
@@ -428,7 +571,7 @@ __global__ __launch_bounds__(256) void lgemm_bf16_kernel(LGemmArgs a) {
     const int wm = wave >> 1, wn = wave & 1;
     f32x16 acc = {}, acc2 = {};
     const int lr = tid >> 2, ks = (tid & 3) * 8;         // this thread stages 8 consecutive k of row lr
-    const bool vecA = (a.lda % 4) == 0 && ((uintptr_t)a.A % 16) == 0;
+    const bool vecA = (a.lda % 4) == 0 && ((uintptr_t)t.A % 16) == 0;
     const bool vecW = (a.K % 8) == 0 && ((uintptr_t)t.W % 16) == 0 && (!DUAL || ((uintptr_t)t.W2 % 16) == 0);
     for (int k0 = 0; k0 < a.K; k0 += BK) {
         const int k = k0 + ks;
@@ -436,11 +579,11 @@ __global__ __launch_bounds__(256) void lgemm_bf16_kernel(LGemmArgs a) {
             float v[8];
             const int ar = arow[lr];
             if (ar >= 0 && vecA && k + 8 <= a.K) {
-                const float4 x0 = *(const float4*)(a.A + (size_t)ar * a.lda + k);
-                const float4 x1 = *(const float4*)(a.A + (size_t)ar * a.lda + k + 4);
+                const float4 x0 = *(const float4*)(t.A + (size_t)ar * a.lda + k);
+                const float4 x1 = *(const float4*)(t.A + (size_t)ar * a.lda + k + 4);
                 v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
             } else {
-                for (int i = 0; i < 8; ++i) v[i] = (ar >= 0 && k + i < a.K) ? a.A[(size_t)ar * a.lda + k + i] : 0.f;
+                for (int i = 0; i < 8; ++i) v[i] = (ar >= 0 && k + i < a.K) ? t.A[(size_t)ar * a.lda + k + i] : 0.f;
             }
             u32x4 pk;
             pk.x = pack_bf16x2(v[0], v[1]); pk.y = pack_bf16x2(v[2], v[3]); pk.z = pack_bf16x2(v[4], v[5]); pk.w = pack_bf16x2(v[6], v[7]);
@@ -487,7 +630,7 @@ __global__ __launch_bounds__(256) void lgemm_bf16_kernel(LGemmArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int r = wm * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-        if (r < t.rows) lg_store(a, t.p0 + r, n, acc[i], acc2[i], DUAL);
+        if (r < t.rows) lg_store(a, t.coff, t.p0 + r, n, acc[i], acc2[i], DUAL);
     }
 }
 
@@ -504,6 +647,8 @@ __global__ __launch_bounds__(256) void lgemv_kernel(LGemmArgs a) {
     rows = min(rows, LV_MAXM);
     const uint16_t* W = a.W + (size_t)g * a.w_stride;
     const uint16_t* W2 = DUAL ? a.W2 + (size_t)g * a.w_stride : nullptr;
+    const float* A = a.A + (a.grp_off ? 0 : (size_t)g * a.a_goff);
+    const size_t coff = a.grp_off ? 0 : (size_t)g * a.c_goff;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = (blockIdx.x * 4 + wave) * 2;
     if (n0 >= a.N) return;
@@ -516,7 +661,7 @@ __global__ __launch_bounds__(256) void lgemv_kernel(LGemmArgs a) {
     }
     float acc[2][LV_MAXM] = {}, acc2[2][LV_MAXM] = {};
     const int K = a.K;
-    const bool vec = (K % 8) == 0 && (a.lda % 4) == 0 && ((uintptr_t)a.A % 16) == 0 && ((uintptr_t)W % 16) == 0 &&
+    const bool vec = (K % 8) == 0 && (a.lda % 4) == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 &&
                      (!DUAL || ((uintptr_t)W2 % 16) == 0);
     if (vec) {
         for (int k = lane * 8; k < K; k += 512) {
@@ -526,7 +671,7 @@ __global__ __launch_bounds__(256) void lgemv_kernel(LGemmArgs a) {
 #pragma unroll
             for (int r = 0; r < LV_MAXM; ++r) {
                 if (r < rows) {
-                    const float4 xa = *(const float4*)(a.A + ar[r] + k), xb = *(const float4*)(a.A + ar[r] + k + 4);
+                    const float4 xa = *(const float4*)(A + ar[r] + k), xb = *(const float4*)(A + ar[r] + k + 4);
                     float x[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
                     if (BF16) {
 #pragma unroll
@@ -551,7 +696,7 @@ __global__ __launch_bounds__(256) void lgemv_kernel(LGemmArgs a) {
 #pragma unroll
             for (int r = 0; r < LV_MAXM; ++r) {
                 if (r < rows) {
-                    float x = a.A[ar[r] + k];
+                    float x = A[ar[r] + k];
                     if (BF16) x = bf16_round(x);
                     acc[0][r] = fmaf(w0, x, acc[0][r]); acc[1][r] = fmaf(w1, x, acc[1][r]);
                     if (DUAL) { acc2[0][r] = fmaf(v0, x, acc2[0][r]); acc2[1][r] = fmaf(v1, x, acc2[1][r]); }
@@ -566,22 +711,22 @@ __global__ __launch_bounds__(256) void lgemv_kernel(LGemmArgs a) {
             for (int c = 0; c < 2; ++c) {
                 const float v = wave_sum(acc[c][r]);
                 const float v2 = DUAL ? wave_sum(acc2[c][r]) : 0.f;
-                if (lane == 0 && (c == 0 || n0 + 1 < a.N)) lg_store(a, base + r, n0 + c, v, v2, DUAL);
+                if (lane == 0 && (c == 0 || n0 + 1 < a.N)) lg_store(a, coff, base + r, n0 + c, v, v2, DUAL);
             }
         }
     }
 }
 
 // the column-range activation of a finished product, in place (products that ran on the shared GEMM kernels)
-__global__ __launch_bounds__(256) void lay_act_cols_kernel(float* __restrict__ C, int ldc, int N, int act, int act2, int split) {
+__global__ __launch_bounds__(256) void lay_act_cols_kernel(float* __restrict__ C, int ldc, int N, int act, int act2, int split, float param) {
     const int n = blockIdx.y * 256 + threadIdx.x;
     if (n >= N) return;
     float* p = C + (size_t)blockIdx.x * ldc + n;
-    *p = lay_act(*p, n < split ? act : act2);
+    *p = lay_act(*p, n < split ? act : act2, param);
 }
-void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int split, hipStream_t s) {
-    if (M <= 0 || (act == LACT_NONE && (act2 == LACT_NONE || split >= N))) return;
-    hipLaunchKernelGGL(lay_act_cols_kernel, dim3((unsigned)M, (unsigned)((N + 255) / 256)), dim3(256), 0, s, C, ldc, N, act, act2, split);
+void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int split, hipStream_t s, float param) {
+    if (M <= 0 || ((act == LACT_NONE || split <= 0) && (act2 == LACT_NONE || split >= N))) return;
+    hipLaunchKernelGGL(lay_act_cols_kernel, dim3((unsigned)M, (unsigned)((N + 255) / 256)), dim3(256), 0, s, C, ldc, N, act, act2, split, param);
 }
 // out = act(g) * u
 __global__ __launch_bounds__(256) void lay_act_mul_kernel(const float* __restrict__ g, const float* __restrict__ u, float* __restrict__ out,
@@ -659,16 +804,22 @@ void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int
 
 // A block = 16 query rows of one sequence and one key head: row qi = (position in the portion) * nrep + (query head in the
 // group), so that a single decode token fills the tile with the heads that share its keys.  16 lanes per query row.
-// Keys the tile can see: the kept first tokens [0, min(keep, lo)) and the window [lo, last position]; each query masks
-// with its own position.  Scores, softmax and the weighted sum are f32.
+// Keys the tile can see: the kept first tokens [0, min(keep, lo)) and the window [lo, last position], lo not before the start of
+// the first query's position block when the mask is chunked; each query masks with its own position.  Values: pages of their own
+// ([..][e]) or the first e elements of the key rows.  A sink adds exp(sink) to the denominator: it is the start value of the running
+// (max, sum) pair of the first split.  Scores, softmax and the weighted sum are f32.
 constexpr int LA_BQ = 16;
-template <int KVT, int KT>
+template <int KVT, int KT, int NACC>
 __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
     extern __shared__ float lds[];
-    const int d = a.d, ldk = d + 1;
+    const int d = a.d, e = a.e, ldk = d + 1;
+    const bool ownv = a.vpool != nullptr;
     float* qs = lds;                       // [16][d]
     float* ks = qs + LA_BQ * d;            // [KT][d + 1]
-    float* ps = ks + KT * ldk;             // [16][KT]
+    float* vs = ks + KT * ldk;             // [KT][e], own value pages only
+    float* ps = vs + (ownv ? KT * e : 0);  // [16][KT]
+    const float* vt = ownv ? vs : ks;
+    const int ldv = ownv ? e : ldk;
     const int2 tile = a.tiles[blockIdx.x];
     const LaySegDev sg = a.segs[tile.x];
     const int g = blockIdx.y, nrep = a.H / a.G;
@@ -679,16 +830,19 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
     const int lp = qi / nrep, head = g * nrep + (qi - lp * nrep);
     const int pos = sg.start_pos + lp;
     const int row = sg.row0 + lp;
-    const int win = (int)min(a.win, 1ll << 30), keep = (int)min(a.keep, 1ll << 30);
+    const int win = (int)min(a.win, 1ll << 30), keep = (int)min(a.keep, 1ll << 30), chunk = (int)min(a.chunk, 1ll << 30);
     for (int i = ln; i < d; i += 16) qs[qr * d + i] = qvalid ? a.proj[(size_t)row * a.ldp + a.q_off + head * d + i] : 0.f;
     const int pmin = sg.start_pos + q0 / nrep, pmax = sg.start_pos + (q0 + nq - 1) / nrep;
-    const int main_lo = max(0, pmin - win + 1);
+    int main_lo = max(0, pmin - win + 1);
+    if (chunk > 0) main_lo = max(main_lo, pmin / chunk * chunk);
+    const int clo = chunk > 0 ? pos / chunk * chunk : 0;       // first position of this query's block
     const int sink_hi = min(keep, main_lo);
     const int total = sink_hi + (pmax - main_lo + 1);
-    const float r1 = a.r1[head], r2 = a.r2[head];
-    float m = -INFINITY, l = 0.f, acc[16];
+    const float r1 = a.bias != LBIAS_NONE ? a.r1[head] : 0.f, r2 = a.bias == LBIAS_LOG ? a.r2[head] : 0.f;
+    float m = -INFINITY, l = 0.f, acc[NACC];
+    if (a.sink && blockIdx.z == 0 && qvalid) { m = a.sink[head]; l = 1.f; }
 #pragma unroll
-    for (int c = 0; c < 16; ++c) acc[c] = 0.f;
+    for (int c = 0; c < NACC; ++c) acc[c] = 0.f;
     const size_t esz = KVT == KV_F32 ? 4 : 2;
     const int nsplit = (int)gridDim.z;     // the visible keys' tiles are dealt round-robin to nsplit blocks (few queries, many keys)
     __syncthreads();                       // qs written (a split may have no tile at all)
@@ -711,8 +865,14 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
                 } else
                 for (int i = ln; i < d; i += 16)
                     ks[sl * ldk + i] = KVT == KV_F32 ? ((const float*)src)[i] : bf16_to_f32(((const uint16_t*)src)[i]);
+                if (ownv) {
+                    const char* vsrc = (const char*)a.vpool + ((((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * e) * esz;
+                    for (int i = ln; i < e; i += 16)
+                        vs[sl * e + i] = KVT == KV_F32 ? ((const float*)vsrc)[i] : bf16_to_f32(((const uint16_t*)vsrc)[i]);
+                }
             } else {
                 for (int i = ln; i < d; i += 16) ks[sl * ldk + i] = 0.f;
+                if (ownv) for (int i = ln; i < e; i += 16) vs[sl * e + i] = 0.f;
             }
         }
         __syncthreads();
@@ -726,8 +886,9 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
             float dot = 0.f;
             for (int i = 0; i < d; ++i) dot = fmaf(qs[qr * d + i], ks[sl * ldk + i], dot);
             const int dist = pos - j;
-            const bool vis = qvalid && v < total && dist >= 0 && (dist < win || j < keep);
-            sc[c] = vis ? dot * a.scale - r1 * log1pf(r2 * (float)dist) : -INFINITY;
+            const bool vis = qvalid && v < total && dist >= 0 && ((dist < win && j >= clo) || j < keep);
+            const float pen = a.bias == LBIAS_LOG ? r1 * log1pf(r2 * (float)dist) : r1 * (float)dist;
+            sc[c] = vis ? dot * a.scale - pen : -INFINITY;
             tmax = fmaxf(tmax, sc[c]);
         }
         tmax = row16_max(tmax);
@@ -746,11 +907,11 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         __syncthreads();
         const int kn = min(KT, total - v0);
 #pragma unroll
-        for (int c = 0; c < 16; ++c) {
+        for (int c = 0; c < NACC; ++c) {
             const int i = ln + 16 * c;
-            if (i < d) {
+            if (i < e) {
                 float o = acc[c] * corr;
-                for (int sl = 0; sl < kn; ++sl) o = fmaf(ps[qr * KT + sl], ks[sl * ldk + i], o);
+                for (int sl = 0; sl < kn; ++sl) o = fmaf(ps[qr * KT + sl], vt[sl * ldv + i], o);
                 acc[c] = o;
             }
         }
@@ -759,19 +920,19 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         const size_t pr = (((size_t)blockIdx.x * a.G + g) * nsplit + blockIdx.z) * LA_BQ + qr;
         if (ln == 0) { a.part_ml[pr * 2] = m; a.part_ml[pr * 2 + 1] = l; }
 #pragma unroll
-        for (int c = 0; c < 16; ++c) {
+        for (int c = 0; c < NACC; ++c) {
             const int i = ln + 16 * c;
-            if (i < d) a.part_o[pr * d + i] = acc[c];
+            if (i < e) a.part_o[pr * e + i] = acc[c];
         }
         return;
     }
     if (!qvalid) return;
-    const float gate = a.proj[(size_t)row * a.ldp + a.g_off + head];
-    const float inv = gate / l;
+    const float* gp = a.proj + (size_t)row * a.ldp + a.g_off + (a.gate == LGATE_ELEM ? head * e : head);
+    const float inv = (a.gate == LGATE_HEAD ? gp[0] : 1.f) / l;
 #pragma unroll
-    for (int c = 0; c < 16; ++c) {
+    for (int c = 0; c < NACC; ++c) {
         const int i = ln + 16 * c;
-        if (i < d) a.out[(size_t)row * a.ldo + head * d + i] = acc[c] * inv;
+        if (i < e) a.out[(size_t)row * a.ldo + head * e + i] = acc[c] * inv * (a.gate == LGATE_ELEM ? gp[i] : 1.f);
     }
 }
 // Matrix-core form for prompt passes in the bfloat16 format (head size a multiple of 16, up to 128): LAY_ATTN_MFMA_ROWS query rows per
@@ -932,7 +1093,7 @@ void launch_lay_attn_mfma(const LAttnArgs& a, hipStream_t s) {
 __global__ __launch_bounds__(256) void lay_attn_merge_kernel(LAttnArgs a, int nsplit) {
     const int2 tile = a.tiles[blockIdx.x];
     const LaySegDev sg = a.segs[tile.x];
-    const int g = blockIdx.y, nrep = a.H / a.G, d = a.d;
+    const int g = blockIdx.y, nrep = a.H / a.G, d = a.e;
     const int q0 = tile.y, nq = min(LA_BQ, sg.n * nrep - q0);
     const size_t t0 = ((size_t)blockIdx.x * a.G + g) * nsplit * LA_BQ;
     for (int idx = threadIdx.x; idx < nq * d; idx += 256) {
@@ -950,22 +1111,48 @@ __global__ __launch_bounds__(256) void lay_attn_merge_kernel(LAttnArgs a, int ns
             L = fmaf(a.part_ml[pr * 2 + 1], w, L);
             acc = fmaf(a.part_o[pr * d + i], w, acc);
         }
-        a.out[(size_t)row * a.ldo + head * d + i] = acc * a.proj[(size_t)row * a.ldp + a.g_off + head] / L;
+        const float gate = a.gate == LGATE_NONE ? 1.f : a.proj[(size_t)row * a.ldp + a.g_off + (a.gate == LGATE_ELEM ? head * d + i : head)];
+        a.out[(size_t)row * a.ldo + head * d + i] = acc * gate / L;
     }
 }
-void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s) {
-    if (a.ntiles <= 0) return;
+static size_t lay_attn_lds(int d, int e, bool own_v, int KT) {
+    return (size_t)(LA_BQ * d + KT * (d + 1) + (own_v ? KT * e : 0) + LA_BQ * KT) * sizeof(float);
+}
+constexpr size_t LDS_PLAIN = 64 * 1024, LDS_MAX = 160 * 1024;    // without / with the kernel's dynamic-LDS attribute raised
+bool lay_attn_fits(int d, int e, bool own_v) {
+    return d > 0 && e > 0 && e <= 512 && (own_v || e <= d) && lay_attn_lds(d, e, own_v, 32) <= LDS_MAX;
+}
+template <int KVT, int KT, int NACC>
+static void lay_attn_go(const LAttnArgs& a, dim3 grid, size_t lds, hipStream_t s) {
+    if (lds > LDS_PLAIN) {
+        static bool raised = false;        // per instantiation
+        if (!raised) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&lay_attn_kernel<KVT, KT, NACC>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)LDS_MAX);
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL((lay_attn_kernel<KVT, KT, NACC>), grid, dim3(256), lds, s, a);
+}
+void launch_lay_attn(const LAttnArgs& a0, int kvt, hipStream_t s) {
+    if (a0.ntiles <= 0) return;
+    LAttnArgs a = a0;
+    if (a.e <= 0) a.e = a.d;               // values = whole key rows
+    const bool own_v = a.vpool != nullptr;
     const int nsplit = (a.part_o && a.part_ml && a.nsplit > 1) ? a.nsplit : 1;
     const dim3 grid((unsigned)a.ntiles, (unsigned)a.G, (unsigned)nsplit);
-    const bool narrow = a.d > 128;         // 32-key tiles keep the block inside 64 KiB of LDS up to d = 256
-    const int KT = narrow ? 32 : 64;
-    const size_t lds = (size_t)(LA_BQ * a.d + KT * (a.d + 1) + LA_BQ * KT) * sizeof(float);
+    // 64-key tiles where they stay inside 64 KiB of LDS (key head sizes up to 128 without value pages of their own), else 32
+    const bool narrow = a.d > 128 || lay_attn_lds(a.d, a.e, own_v, 64) > LDS_PLAIN;
+    const size_t lds = lay_attn_lds(a.d, a.e, own_v, narrow ? 32 : 64);
+    const bool wide = a.e > 256;           // 32 output elements per lane instead of 16
     if (kvt == KV_F32) {
-        if (narrow) hipLaunchKernelGGL((lay_attn_kernel<KV_F32, 32>), grid, dim3(256), lds, s, a);
-        else hipLaunchKernelGGL((lay_attn_kernel<KV_F32, 64>), grid, dim3(256), lds, s, a);
+        if (wide) lay_attn_go<KV_F32, 32, 32>(a, grid, lds, s);
+        else if (narrow) lay_attn_go<KV_F32, 32, 16>(a, grid, lds, s);
+        else lay_attn_go<KV_F32, 64, 16>(a, grid, lds, s);
     } else {
-        if (narrow) hipLaunchKernelGGL((lay_attn_kernel<KV_BF16, 32>), grid, dim3(256), lds, s, a);
-        else hipLaunchKernelGGL((lay_attn_kernel<KV_BF16, 64>), grid, dim3(256), lds, s, a);
+        if (wide) lay_attn_go<KV_BF16, 32, 32>(a, grid, lds, s);
+        else if (narrow) lay_attn_go<KV_BF16, 32, 16>(a, grid, lds, s);
+        else lay_attn_go<KV_BF16, 64, 16>(a, grid, lds, s);
     }
     if (nsplit > 1) hipLaunchKernelGGL(lay_attn_merge_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(256), 0, s, a, nsplit);
 }
@@ -977,6 +1164,20 @@ void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s) {
 // (t, s local to the chunk of n tokens).  Everything is f32.
 // ------------------------------------------------------------------------------------------------------------------
 constexpr int LL_ES = 32;
+// GT (gated form): the decay of key channel i at token t is exp(ldec[t][head d + i]) instead of the head's constant.  With
+// b_t = sum of the logarithms up to and including t (inside the chunk), all factors are exponentials of differences <= 0:
+//   o_t = S0^T (q_t * e^(b_t)) + sum_(s <= t) (sum_i q_t[i] k_s[i] e^(b_t[i] - b_s[i])) v_s,   S <- diag(e^(b_(n-1))) S0 + sum_s (k_s * e^(b_(n-1) - b_s)) v_s^T
+// LDS of the gated form: one more [C][d] array (the running logarithms)
+template <bool GT>
+__device__ __forceinline__ void ll_cumsum(float* bs, int n, int d, int tid) {
+    if (GT) {
+        for (int i = tid; i < d; i += 256) {
+            float run = 0.f;
+            for (int t = 0; t < n; ++t) { run += bs[t * d + i]; bs[t * d + i] = run; }
+        }
+    }
+}
+template <bool GT>
 __global__ __launch_bounds__(256) void lay_lightning_kernel(LLightArgs a, int C) {
     extern __shared__ float lds[];
     const int d = a.d, e = a.e;
@@ -986,53 +1187,69 @@ __global__ __launch_bounds__(256) void lay_lightning_kernel(LLightArgs a, int C)
     float* vs = ks + C * d;                // [C][ES]
     float* As = vs + C * LL_ES;            // [C][C]
     float* pw = As + C * C;                // [C + 1] decay^n
+    float* bs = pw + C + 1;                // gated: [C][d]
     const LaySegDev sg = a.segs[blockIdx.x];
     const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
     const int ne = min(LL_ES, e - j0);
-    const float decay = a.decay[head];
+    const float decay = GT ? 1.f : a.decay[head];
     float* st = a.state_pool + (size_t)sg.slot * a.slot_stride + a.st_off + (size_t)head * d * e;
     for (int idx = tid; idx < d * LL_ES; idx += 256) {
         const int i = idx / LL_ES, j = idx % LL_ES;
         S[idx] = j < ne ? st[(size_t)i * e + j0 + j] : 0.f;
     }
-    if (tid <= C) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
+    if (!GT && tid <= C) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
     for (int t0 = 0; t0 < sg.n; t0 += C) {
         const int n = min(C, sg.n - t0);
         __syncthreads();                   // S, pw ready; the previous chunk's q / k / v no longer read
         for (int idx = tid; idx < n * d; idx += 256) {
             const int t = idx / d, i = idx - t * d;
             const size_t base = (size_t)(sg.row0 + t0 + t) * a.ldp + (size_t)head * d + i;
-            qs[idx] = a.proj[base + a.q_off];
+            qs[idx] = a.proj[base + a.q_off] * a.qscale;
             ks[idx] = a.proj[base + a.k_off];
+            if (GT) bs[idx] = a.ldec[(size_t)(sg.row0 + t0 + t) * a.ldd + (size_t)head * d + i];
         }
         for (int idx = tid; idx < n * LL_ES; idx += 256) {
             const int t = idx / LL_ES, j = idx % LL_ES;
             vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + t0 + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
         }
+        if (GT) { __syncthreads(); ll_cumsum<GT>(bs, n, d, tid); }
         __syncthreads();
         for (int idx = tid; idx < n * n; idx += 256) {
             const int t = idx / n, s = idx - t * n;
             float dot = 0.f;
             if (s <= t) {
-                for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * d + i], dot);
-                dot *= pw[t - s];
+                if (GT) {
+                    for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i] * ks[s * d + i], expf(bs[t * d + i] - bs[s * d + i]), dot);
+                } else {
+                    for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * d + i], dot);
+                    dot *= pw[t - s];
+                }
             }
             As[t * C + s] = dot;
         }
         __syncthreads();
+        if (GT) {                          // q_t e^(b_t) and k_s e^(b_(n-1) - b_s) in place: what the state terms need
+            for (int idx = tid; idx < n * d; idx += 256) {
+                const int i = idx % d;
+                qs[idx] *= expf(bs[idx]);
+                ks[idx] *= expf(bs[(n - 1) * d + i] - bs[idx]);
+            }
+            __syncthreads();
+        }
         for (int idx = tid; idx < n * LL_ES; idx += 256) {
             const int t = idx / LL_ES, j = idx % LL_ES;
             float inter = 0.f;
             for (int i = 0; i < d; ++i) inter = fmaf(S[i * LL_ES + j], qs[t * d + i], inter);
-            float o = inter * pw[t + 1];
+            float o = GT ? inter : inter * pw[t + 1];
             for (int s = 0; s <= t; ++s) o = fmaf(As[t * C + s], vs[s * LL_ES + j], o);
             if (j < ne) a.out[(size_t)(sg.row0 + t0 + t) * a.ldo + (size_t)head * e + j0 + j] = o;
         }
         __syncthreads();
         for (int idx = tid; idx < d * LL_ES; idx += 256) {
             const int i = idx / LL_ES, j = idx % LL_ES;
-            float sv = S[idx] * pw[n];
-            for (int s = 0; s < n; ++s) sv = fmaf(pw[n - 1 - s] * ks[s * d + i], vs[s * LL_ES + j], sv);
+            float sv = S[idx] * (GT ? expf(bs[(n - 1) * d + i]) : pw[n]);
+            if (GT) { for (int s = 0; s < n; ++s) sv = fmaf(ks[s * d + i], vs[s * LL_ES + j], sv); }
+            else for (int s = 0; s < n; ++s) sv = fmaf(pw[n - 1 - s] * ks[s * d + i], vs[s * LL_ES + j], sv);
             S[idx] = sv;
         }
     }
@@ -1044,58 +1261,78 @@ __global__ __launch_bounds__(256) void lay_lightning_kernel(LLightArgs a, int C)
 }
 // Long portions: the same recurrence in three launches that are parallel over chunks of LC tokens.
 //   1. every chunk's own contribution  U_c = sum_s decay^(n-1-s) k_s v_s^T                        (chunk, head, value slice)
+//      (gated: also D_c = e^(b_(n-1)), the decay of the whole chunk per key channel)
 //   2. the states in front of the chunks by a scan over each sequence's chunks, in place: U_c <- S_c, S_(c+1) = decay^n S_c + U_c,
 //      last state back to the pool                                                              (sequence, head, state element)
 //   3. o_t = decay^(t+1) S_c^T q_t + sum_(s <= t) decay^(t-s) (q_t . k_s) v_s                      (chunk, head, value slice)
 // chunks[c] = {segment, first token of the chunk inside the portion}; a segment's chunks are consecutive, the first is segs[].pad0.
 constexpr int LC = 32;
+template <bool GT>
 __global__ __launch_bounds__(256) void lay_light_chunk_kv_kernel(LLightArgs a) {
     extern __shared__ float lds[];
     const int d = a.d, e = a.e;
     float* ks = lds;                       // [LC][d]
     float* vs = ks + LC * d;               // [LC][ES]
     float* pw = vs + LC * LL_ES;           // [LC + 1]
+    float* bs = pw + LC + 1;               // gated: [LC][d]
     const int2 ch = a.chunks[blockIdx.x];
     const LaySegDev sg = a.segs[ch.x];
     const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
     const int ne = min(LL_ES, e - j0), n = min(LC, sg.n - ch.y);
-    const float decay = a.decay[head];
-    if (tid <= LC) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
+    if (!GT) {
+        const float decay = a.decay[head];
+        if (tid <= LC) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
+    }
     for (int idx = tid; idx < n * d; idx += 256) {
         const int t = idx / d, i = idx - t * d;
         ks[idx] = a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.k_off + (size_t)head * d + i];
+        if (GT) bs[idx] = a.ldec[(size_t)(sg.row0 + ch.y + t) * a.ldd + (size_t)head * d + i];
     }
     for (int idx = tid; idx < n * LL_ES; idx += 256) {
         const int t = idx / LL_ES, j = idx % LL_ES;
         vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
     }
     __syncthreads();
+    if (GT) {
+        ll_cumsum<GT>(bs, n, d, tid);
+        __syncthreads();
+        for (int idx = tid; idx < n * d; idx += 256) ks[idx] *= expf(bs[(n - 1) * d + idx % d] - bs[idx]);
+        if (blockIdx.z == 0) for (int i = tid; i < d; i += 256) a.D[((size_t)blockIdx.x * a.H + head) * d + i] = expf(bs[(n - 1) * d + i]);
+        __syncthreads();
+    }
     float* U = a.U + ((size_t)blockIdx.x * a.H + head) * d * e;
     for (int idx = tid; idx < d * LL_ES; idx += 256) {
         const int i = idx / LL_ES, j = idx % LL_ES;
         float sv = 0.f;
-        for (int s = 0; s < n; ++s) sv = fmaf(pw[n - 1 - s] * ks[s * d + i], vs[s * LL_ES + j], sv);
+        if (GT) { for (int s = 0; s < n; ++s) sv = fmaf(ks[s * d + i], vs[s * LL_ES + j], sv); }
+        else for (int s = 0; s < n; ++s) sv = fmaf(pw[n - 1 - s] * ks[s * d + i], vs[s * LL_ES + j], sv);
         if (j < ne) U[(size_t)i * e + j0 + j] = sv;
     }
 }
+template <bool GT>
 __global__ __launch_bounds__(256) void lay_light_scan_kernel(LLightArgs a) {
     const LaySegDev sg = a.segs[blockIdx.x];
     const int head = blockIdx.y, de = a.d * a.e;
     const int el = blockIdx.z * 256 + threadIdx.x;
     if (el >= de) return;
-    const float decay = a.decay[head];
     const int nch = (sg.n + LC - 1) / LC;
-    const float pfull = powf(decay, (float)LC), plast = powf(decay, (float)(sg.n - (nch - 1) * LC));
+    float pfull = 1.f, plast = 1.f;
+    if (!GT) {
+        const float decay = a.decay[head];
+        pfull = powf(decay, (float)LC); plast = powf(decay, (float)(sg.n - (nch - 1) * LC));
+    }
     float* st = a.state_pool + (size_t)sg.slot * a.slot_stride + a.st_off + (size_t)head * de + el;
     float S = *st;
     for (int c = 0; c < nch; ++c) {
         float* u = a.U + ((size_t)(sg.pad0 + c) * a.H + head) * de + el;
         const float own = *u;
         *u = S;
-        S = fmaf(S, c == nch - 1 ? plast : pfull, own);
+        const float dc = GT ? a.D[((size_t)(sg.pad0 + c) * a.H + head) * a.d + el / a.e] : (c == nch - 1 ? plast : pfull);
+        S = fmaf(S, dc, own);
     }
     *st = S;
 }
+template <bool GT>
 __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) {
     extern __shared__ float lds[];
     const int d = a.d, e = a.e;
@@ -1106,12 +1343,15 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
     float* vs = ks + LC * ldk;             // [LC][ES]
     float* As = vs + LC * LL_ES;           // [LC][LC]
     float* pw = As + LC * LC;              // [LC + 1]
+    float* bs = pw + LC + 1;               // gated: [LC][d + 1]
     const int2 ch = a.chunks[blockIdx.x];
     const LaySegDev sg = a.segs[ch.x];
     const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
     const int ne = min(LL_ES, e - j0), n = min(LC, sg.n - ch.y);
-    const float decay = a.decay[head];
-    if (tid <= LC) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
+    if (!GT) {
+        const float decay = a.decay[head];
+        if (tid <= LC) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
+    }
     const float* U = a.U + ((size_t)blockIdx.x * a.H + head) * d * e;
     for (int idx = tid; idx < d * LL_ES; idx += 256) {
         const int i = idx / LL_ES, j = idx % LL_ES;
@@ -1120,29 +1360,45 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
     for (int idx = tid; idx < n * d; idx += 256) {
         const int t = idx / d, i = idx - t * d;
         const size_t base = (size_t)(sg.row0 + ch.y + t) * a.ldp + (size_t)head * d + i;
-        qs[idx] = a.proj[base + a.q_off];
+        qs[idx] = a.proj[base + a.q_off] * a.qscale;
         ks[t * ldk + i] = a.proj[base + a.k_off];
+        if (GT) bs[t * ldk + i] = a.ldec[(size_t)(sg.row0 + ch.y + t) * a.ldd + (size_t)head * d + i];
     }
     for (int idx = tid; idx < n * LL_ES; idx += 256) {
         const int t = idx / LL_ES, j = idx % LL_ES;
         vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
     }
     __syncthreads();
+    if (GT) {
+        for (int i = tid; i < d; i += 256) {
+            float run = 0.f;
+            for (int t = 0; t < n; ++t) { run += bs[t * ldk + i]; bs[t * ldk + i] = run; }
+        }
+        __syncthreads();
+    }
     for (int idx = tid; idx < n * n; idx += 256) {
         const int t = idx / n, s = idx - t * n;
         float dot = 0.f;
         if (s <= t) {
-            for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * ldk + i], dot);
-            dot *= pw[t - s];
+            if (GT) {
+                for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i] * ks[s * ldk + i], expf(bs[t * ldk + i] - bs[s * ldk + i]), dot);
+            } else {
+                for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * ldk + i], dot);
+                dot *= pw[t - s];
+            }
         }
         As[t * LC + s] = dot;
     }
     __syncthreads();
+    if (GT) {
+        for (int idx = tid; idx < n * d; idx += 256) { const int t = idx / d, i = idx - t * d; qs[idx] *= expf(bs[t * ldk + i]); }
+        __syncthreads();
+    }
     for (int idx = tid; idx < n * LL_ES; idx += 256) {
         const int t = idx / LL_ES, j = idx % LL_ES;
         float inter = 0.f;
         for (int i = 0; i < d; ++i) inter = fmaf(S[i * LL_ES + j], qs[t * d + i], inter);
-        float o = inter * pw[t + 1];
+        float o = GT ? inter : inter * pw[t + 1];
         for (int s = 0; s <= t; ++s) o = fmaf(As[t * LC + s], vs[s * LL_ES + j], o);
         if (j < ne) a.out[(size_t)(sg.row0 + ch.y + t) * a.ldo + (size_t)head * e + j0 + j] = o;
     }
@@ -1150,18 +1406,20 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
 
 // single-token portions (decode steps): S <- decay S + k v^T and o = S^T q straight on the state in HBM, no staging; thread =
 // (value column j, 1/8 of the key rows); the eight partial sums of a column meet in LDS
+template <bool GT>
 __global__ __launch_bounds__(256) void lay_light_decode_kernel(LLightArgs a) {
-    __shared__ float qk[2 * 256];
+    __shared__ float qk[3 * 256];
     __shared__ float part[8][LL_ES];
     const int d = a.d, e = a.e;
     const LaySegDev sg = a.segs[blockIdx.x];
     const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
     const int j = tid & (LL_ES - 1), rg = tid >> 5;
-    const float decay = a.decay[head];
+    const float decay = GT ? 1.f : a.decay[head];
     const size_t prow = (size_t)sg.row0 * a.ldp;
     for (int i = tid; i < d; i += 256) {
-        qk[i] = a.proj[prow + a.q_off + (size_t)head * d + i];
+        qk[i] = a.proj[prow + a.q_off + (size_t)head * d + i] * a.qscale;
         qk[256 + i] = a.proj[prow + a.k_off + (size_t)head * d + i];
+        if (GT) qk[512 + i] = expf(a.ldec[(size_t)sg.row0 * a.ldd + (size_t)head * d + i]);
     }
     __syncthreads();
     const bool ok = j0 + j < e;
@@ -1170,7 +1428,7 @@ __global__ __launch_bounds__(256) void lay_light_decode_kernel(LLightArgs a) {
     float o = 0.f;
     if (ok)
         for (int i = rg; i < d; i += 8) {
-            const float sv = fmaf(st[(size_t)i * e], decay, qk[256 + i] * v);
+            const float sv = fmaf(st[(size_t)i * e], GT ? qk[512 + i] : decay, qk[256 + i] * v);
             st[(size_t)i * e] = sv;
             o = fmaf(sv, qk[i], o);
         }
@@ -1184,24 +1442,34 @@ __global__ __launch_bounds__(256) void lay_light_decode_kernel(LLightArgs a) {
     }
 }
 
-void launch_lay_lightning(const LLightArgs& a, hipStream_t s) {
-    if (a.nseg <= 0) return;
+template <typename K>
+static void ll_raise_lds(K kern, size_t lds) {
+    if (lds > LDS_PLAIN) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
+}
+template <bool GT>
+static void lay_lightning_go(const LLightArgs& a, hipStream_t s) {
     if (a.all_single && a.d <= 256) {
-        hipLaunchKernelGGL(lay_light_decode_kernel, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES)), dim3(256), 0, s, a);
+        hipLaunchKernelGGL(lay_light_decode_kernel<GT>, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES)), dim3(256), 0, s, a);
         return;
     }
-    if (a.U && a.chunks && a.nchunks > 0 && a.d <= 128) {
+    if (a.U && a.chunks && a.nchunks > 0 && a.d <= 128 && (!GT || a.D)) {
         const dim3 gc((unsigned)a.nchunks, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES));
-        const size_t l1 = (size_t)(LC * a.d + LC * LL_ES + LC + 1) * sizeof(float);
-        const size_t l3 = (size_t)(a.d * LL_ES + 2 * LC * a.d + LC + LC * LL_ES + LC * LC + LC + 1) * sizeof(float);
-        hipLaunchKernelGGL(lay_light_chunk_kv_kernel, gc, dim3(256), l1, s, a);
-        hipLaunchKernelGGL(lay_light_scan_kernel, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.d * a.e + 255) / 256)), dim3(256), 0, s, a);
-        hipLaunchKernelGGL(lay_light_chunk_out_kernel, gc, dim3(256), l3, s, a);
+        const size_t l1 = (size_t)(LC * a.d + LC * LL_ES + LC + 1 + (GT ? LC * a.d : 0)) * sizeof(float);
+        const size_t l3 = (size_t)(a.d * LL_ES + 2 * LC * a.d + LC + LC * LL_ES + LC * LC + LC + 1 + (GT ? LC * (a.d + 1) : 0)) * sizeof(float);
+        ll_raise_lds(lay_light_chunk_out_kernel<GT>, l3);
+        hipLaunchKernelGGL(lay_light_chunk_kv_kernel<GT>, gc, dim3(256), l1, s, a);
+        hipLaunchKernelGGL(lay_light_scan_kernel<GT>, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.d * a.e + 255) / 256)), dim3(256), 0, s, a);
+        hipLaunchKernelGGL(lay_light_chunk_out_kernel<GT>, gc, dim3(256), l3, s, a);
         return;
     }
     const int C = a.d > 128 ? 8 : 16;
-    const size_t lds = (size_t)(a.d * LL_ES + 2 * C * a.d + C * LL_ES + C * C + C + 1) * sizeof(float);
-    hipLaunchKernelGGL(lay_lightning_kernel, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES)), dim3(256), lds, s, a, C);
+    const size_t lds = (size_t)(a.d * LL_ES + 2 * C * a.d + C * LL_ES + C * C + C + 1 + (GT ? C * a.d : 0)) * sizeof(float);
+    hipLaunchKernelGGL(lay_lightning_kernel<GT>, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.e + LL_ES - 1) / LL_ES)), dim3(256), lds, s, a, C);
+}
+void launch_lay_lightning(const LLightArgs& a, hipStream_t s) {
+    if (a.nseg <= 0) return;
+    if (a.ldec) lay_lightning_go<true>(a, s);
+    else lay_lightning_go<false>(a, s);
 }
 
 // ------------------------------------------------------------------------------------------------------------------

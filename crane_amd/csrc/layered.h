@@ -1,9 +1,15 @@
 // Layer-list decoders: a model whose config.json spells out every layer (mixer kind + sizes, feed-forward kind + sizes) instead
-// of a family-wide geometry.  First member: Korupel (sandwich RMS norms with a scaled residual, a short causal convolution in front
-// of every sublayer, softmax attention over a sliding window with kept first tokens / a logarithmic distance penalty / values that
-// are the keys / one sigmoid gate per head, lightning (decayed linear) attention, dense GELU or sigmoid-routed mixture-of-experts
-// feed-forwards).  The mechanisms are kernels with their constants as arguments (kernels_layered.hip); the per-layer plumbing and
-// the step function over mixed batches (prompt portions beside single decode tokens) are in model_layered.cpp.
+// of a family-wide geometry.  Members:
+//   Korupel -- sandwich RMS norms with a scaled residual, a short causal convolution in front of every sublayer, softmax attention
+//     over a sliding window with kept first tokens / a logarithmic distance penalty / values that are the keys / one sigmoid gate
+//     per head, lightning (decayed linear) attention, dense GELU or sigmoid-routed mixture-of-experts feed-forwards;
+//   Mononex -- mixer and feed-forward in parallel on two norms of the same residual (weights stored around zero), a token shift in
+//     front of the mixer (the two-tap case of the short convolution), softmax attention inside position chunks with a linear
+//     distance bias / a sink term in the denominator / an element-wise sigmoid gate / keys and values borrowed from an earlier
+//     layer, latent attention (low-rank queries, one cached latent + one rotated key part per token, YaRN-scaled rotation), gated
+//     linear attention with a data-dependent decay per key channel, dense squared-ReLU feed-forwards.
+// The mechanisms are kernels with their constants as arguments (kernels_layered.hip); the per-layer plumbing and the step function
+// over mixed batches (prompt portions beside single decode tokens) are in model_layered.cpp.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -13,9 +19,22 @@
 
 namespace cm {
 
-enum { LMIX_ATTN = 0, LMIX_LIGHTNING = 1 };
+enum { LMIX_ATTN = 0, LMIX_LIGHTNING = 1, LMIX_LATENT = 2, LMIX_GLA = 3 };
 enum { LMLP_NONE = 0, LMLP_DENSE = 1, LMLP_MOE = 2 };
-enum { LACT_NONE = 0, LACT_SILU = 1, LACT_SIGMOID = 2, LACT_GELU_TANH = 3 };
+// LACT_RELU2: max(v, 0)^2;  LACT_LOGSIG: act_param * ln(sigmoid(v)) (the logarithm of a decay sigmoid(v)^act_param)
+enum { LACT_NONE = 0, LACT_SILU = 1, LACT_SIGMOID = 2, LACT_GELU_TANH = 3, LACT_RELU2 = 4, LACT_LOGSIG = 5 };
+// distance term taken off an attention score: none | r1 ln(1 + r2 (i - j)) | r1 (i - j)
+enum { LBIAS_NONE = 0, LBIAS_LOG = 1, LBIAS_LINEAR = 2 };
+// gate on the attention output: none | one value per head at g_off + head | one per element at g_off + head e + i
+enum { LGATE_NONE = 0, LGATE_HEAD = 1, LGATE_ELEM = 2 };
+
+// rotation of consecutive pairs (2i, 2i + 1) of the first `dims` elements of a vector by the angle position * freq[i]
+struct RotSpec {
+    int dims = 0;
+    double base = 10000.0;
+    bool yarn = false;
+    double factor = 1.0, original = 0.0, fast = 32.0, slow = 1.0;
+};
 
 // one entry of config "layers"
 struct LayerSpec {
@@ -24,7 +43,17 @@ struct LayerSpec {
     float scale = 1.f;                 // attention: score multiplier
     long long win = 0, keep = 0;       // attention: window size, kept first tokens
     std::vector<float> decay;          // lightning: per head
+    long long chunk = 0;               // attention: positions see each other only inside the same block of `chunk` positions (0: off)
+    int bias = LBIAS_NONE, gate = LGATE_NONE;
+    bool sink = false, own_v = false;  // attention: learned sink per head in the softmax denominator; value projection of its own
+    int kv_from = -1;                  // attention: keys and values of that earlier layer's cache instead of own projections
+    int q_rank = 0, kv_rank = 0, rot_dim = 0;   // latent attention
+    RotSpec rot;
+    float tau = 1.f;                   // gated linear attention: decay = sigmoid(z)^(1 / tau)
+    int a_rank = 0;                    // ... inner size of the decay's low-rank projection (from the checkpoint)
     int mlp = LMLP_NONE, ff = 0, experts = 0, top = 0;
+    bool gated_ff = true;              // dense: act(gate) * up (false: act(up) alone)
+    int ff_act = LACT_GELU_TANH;
 };
 
 // device-side weights of one layer (bf16 matrices [out, in], f32 vectors)
@@ -34,8 +63,18 @@ struct LayeredLayerW {
     // mixer input projection, rows concatenated so that one GEMM produces them:
     //   attention: q (H d) | k (G d) | g (H);  lightning: q (H d) | k (H d) | v (H e) | g (H e)
     uint16_t* in_w = nullptr;
+    //   chunk attention: q (H d) | k (G d) | v (G e) | g (H e) (k, v absent when borrowed);  latent: dq (q_rank) | dkv (kv_rank + rot) | g (H e)
+    //   gated linear attention: q (H d) | k (H d) | v (H e) | a1 (rank) | g (H e)
     float* in_b = nullptr;                           // [rows] (zeros where the checkpoint has no bias) or null
-    int in_rows = 0, q_off = 0, k_off = 0, v_off = 0, g_off = 0;
+    int in_rows = 0, q_off = 0, k_off = 0, v_off = 0, g_off = 0, a_off = 0;
+    float* shift = nullptr;                          // token shift as a two-tap convolution: [W][2] = {s, -s}
+    float *sink = nullptr;                           // attention: [H]
+    float *dq_norm = nullptr, *dkv_norm = nullptr;   // latent attention: plain norm weights of the two latents
+    uint16_t *uq = nullptr, *uk_t = nullptr, *uv = nullptr;   // [H (d + rot)][q_rank]; per head [kv_rank][d] (transposed); [H e][kv_rank]
+    float* rot_freq = nullptr; float rot_mag = 1.f;  // [rot.dims / 2] angle per position; factor on cos and sin
+    uint16_t* a2 = nullptr; float* a2_b = nullptr;   // gated linear attention: [H d][rank], [H d]
+    size_t v_pool_off = 0, v_page_bytes = 0;         // value pages (layers whose values are not their keys)
+    size_t sh_off = 0;                               // the shift's previous input inside a slot of the conv pool (floats)
     uint16_t* o_w = nullptr;                         // [W][H e]
     float *r1 = nullptr, *r2 = nullptr;              // attention: per-head distance penalty
     float* decay = nullptr;                          // lightning: per head
@@ -63,16 +102,35 @@ struct LGemmArgs {
     int M = 0, N = 0, K = 0;
     const int32_t* grp_off = nullptr;                // grouped: rows [grp_off[g], grp_off[g + 1]) use matrix g; M bounds a group's rows
     int act = LACT_NONE, act2 = LACT_NONE, act_split = 0;   // columns < act_split: act, the others act2 (W2: act on the first product)
+    float act_param = 1.f;                           // LACT_LOGSIG: the factor
+    // groups without grp_off (one product per head over all rows): group g reads A + g a_goff, writes C + g c_goff
+    size_t a_goff = 0, c_goff = 0;
+    const float* mul = nullptr; int ldm = 0;         // C[p][n] *= mul[p ldm + g c_goff + n] after the activation
 };
 // bf16 = true: A rounded to bfloat16, matrix cores, f32 accumulation; false: f32 FMA throughout.  Up to 8 rows (per group): the
 // streaming row kernel instead of tiles.
 void launch_lgemm(const LGemmArgs& a, bool bf16, int groups, hipStream_t s);
 
-void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int split, hipStream_t s);
+void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int split, hipStream_t s, float param = 1.f);
 void launch_lay_act_mul(const float* g, const float* u, float* out, size_t n, int act, hipStream_t s);
 void launch_lay_round_rows(const float* x, int ldx, uint16_t* out, int M, int K, hipStream_t s);
 void launch_lay_embed_rows(const uint16_t* emb, const uint32_t* ids, float* x, int T, int W, int V, hipStream_t s);
 void launch_lay_rms_rows(const float* x, const int32_t* rows, const float* w, float* out, int n_rows, int W, float eps, hipStream_t s);
+// two norms of the same rows (one root mean square, two weights)
+void launch_lay_rms_rows2(const float* x, const float* w1, const float* w2, float* out1, float* out2, int T, int W, float eps, hipStream_t s);
+// RMS norm of the column range [off, off + n) of every row: dst[r ldd + c] = src[r lds + off + c] / rms * w[c] (dst may be src + off)
+void launch_lay_rms_cols(const float* src, int lds, int off, int n, const float* w, float* dst, int ldd, int T, float eps, hipStream_t s);
+// single-token rows only (every segment n = 1), one launch: x += y1 + y2 (when y1 is given), out1 = shift(x / rms * w1) with the
+// shift's state (the previous input, in conv_pool) replaced, out2 = x / rms * w2 (when out2 is given).  cw: [W][2] = {s, -s}
+void launch_lay_add_norm2_shift_decode(float* x, const float* y1, const float* y2, const float* w1, const float* w2, float eps, float* out1,
+                                       float* out2, const float* cw, float* conv_pool, size_t slot_stride, size_t off, const LaySegDev* segs,
+                                       int T, int W, hipStream_t s);
+// x += y1 + y2 (y2 may be null)
+void launch_lay_add_rows(float* x, const float* y1, const float* y2, size_t n, hipStream_t s);
+// pairs (2i, 2i + 1), i < dims / 2, of `nvec` vectors per row (vector v at src + r lds + v vstride) turned by position * freq[i];
+// cos and sin times mag; elements past dims are copied.  dst may be src.
+void launch_lay_rope(const float* src, int lds, int s_vstride, float* dst, int ldd, int d_vstride, int nvec, int len, int dims,
+                     const float* freq, float mag, const LaySegDev* segs, const int32_t* rowseg, int T, hipStream_t s);
 // out = h + conv(h) over time per channel; the taps - 1 inputs before a portion come from the sequence's tail in conv_pool
 void launch_lay_canon(const float* h, float* out, const float* cw, const float* conv_pool, size_t slot_stride, size_t off,
                       const LaySegDev* segs, const int32_t* rowseg, int T, int W, int taps, hipStream_t s);
@@ -97,6 +155,10 @@ struct LAttnArgs {
     const float *r1, *r2;
     int H, G, d, page;
     float scale; long long win, keep;
+    long long chunk = 0;                             // > 0: only keys of the query's own block of `chunk` positions
+    int bias = LBIAS_LOG, gate = LGATE_HEAD;
+    const float* sink = nullptr;                     // [H]: exp(sink) joins the denominator once, with no value
+    const void* vpool = nullptr; int e = 0;          // [n_pages][G][page][e]; null: the values are the first e elements of the keys
     // few query tiles, many keys (decode steps): nsplit blocks per tile share its key tiles and a merge launch follows;
     // part_o [ntiles][G][nsplit][16][d], part_ml [ntiles][G][nsplit][16][2].  nsplit <= 1 or null scratch: one block per tile
     int nsplit = 1; float* part_o = nullptr; float* part_ml = nullptr;
@@ -104,6 +166,7 @@ struct LAttnArgs {
 void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int kvt, const int32_t* bt, const LaySegDev* segs,
                          const int32_t* rowseg, int T, int G, int d, int page, hipStream_t s);
 void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s);    // kvt: KV_BF16 | KV_F32
+bool lay_attn_fits(int d, int e, bool own_v);                         // sizes the kernel can hold in LDS and registers
 // bf16 key pages, d % 16 == 0, d <= 128: the matrix-core form; a.tiles lists {segment, first query row} in steps of
 // LAY_ATTN_MFMA_ROWS rows, longest key range first
 constexpr int LAY_ATTN_MFMA_ROWS = 64;
@@ -120,11 +183,17 @@ struct LLightArgs {
     // chunk, U = [nchunks][H][d][e] f32 scratch.  Null / 0: one block per (sequence, head, value slice) walks the portion.
     float* U = nullptr; const int2* chunks = nullptr; int nchunks = 0;
     bool all_single = false;     // every portion of the pass is one token (decode steps): the state is updated in place in HBM
+    // gated form: the decay of key channel i at token t is exp(ldec[t ldd + head d + i]) instead of decay[head]
+    const float* ldec = nullptr; int ldd = 0;
+    float qscale = 1.f;          // q is multiplied by this
+    float* D = nullptr;          // gated chunk-parallel form: [nchunks][H][d] decay of a whole chunk
 };
 constexpr int LAY_LIGHT_CHUNK = 32;
 void launch_lay_lightning(const LLightArgs& a, hipStream_t s);
-// out = o / rms(o) * w * gate over whole rows (gate already passed through the sigmoid)
-void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s);
+// out = o / rms(o) * w * gate (gate already activated).  The root mean square is taken over groups of `group` columns (0: the
+// whole row) and group g's column c uses w[c] (weights shared by the groups) or w[g group + c] (shared_w false).
+void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s,
+                         int group = 0, bool shared_w = false);
 
 // router: z = h . Wr^T in f32, the `top` largest (lowest index first among equals) -> sel [T top], wsel = sigmoid(z)
 void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s);

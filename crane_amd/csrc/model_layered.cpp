@@ -22,6 +22,10 @@ struct Layered {
     std::vector<LayeredLayerW> w;
     int taps = 0;                      // 0: no convolution in front of the sublayers
     float mult = 1.f;
+    // Mononex: x += mixer(shift(norm1 x)) + ff(norm2 x), no norm behind the sublayers; Korupel: one sublayer after the other,
+    // a norm on each side
+    bool parallel = false;
+    int max_q = 0, max_qa = 0, max_cq = 0, max_ld = 0, max_e = 0;
     bool f32 = false;                  // number format of the projections and the key cache
     float* final_norm = nullptr;
     uint16_t* head = nullptr;
@@ -44,6 +48,10 @@ struct Layered {
     float *G1 = nullptr, *G2 = nullptr;   // [cap][widest dense ff] the two products of a gated feed-forward
     float* U = nullptr;                // lightning attention, chunk-parallel form: [chunks of a pass][widest H d e] f32
     size_t u_stride = 0;
+    float* Dch = nullptr;              // gated linear attention, chunk-parallel form: [chunks of a pass][widest H d] decay of a chunk
+    float *H2 = nullptr, *Y2 = nullptr;                  // parallel layers: second norm's rows, feed-forward output
+    float *CQ = nullptr, *Q = nullptr, *Qa = nullptr;    // latent attention: query latent, queries, queries against the cached latent
+    float* LD = nullptr;               // gated linear attention: logarithm of the decay per token and key channel
     static constexpr int ATT_PARTS = 512;   // (query tile, key head, split) blocks of a split-key attention launch
     float *att_po = nullptr, *att_pml = nullptr;
     float* am_pv = nullptr; int* am_pi = nullptr;   // arg-max partials of the logits rows
@@ -61,7 +69,7 @@ void LayeredDeleter::operator()(Layered* p) const { delete p; }
 // one projection of a pass: the shared matrix-core GEMM where it applies, else the kernels of kernels_layered.hip
 static void lay_gemm(Model& m, Layered& L, const LGemmArgs& g, int groups, hipStream_t s) {
     const bool bf = !L.f32;
-    if (bf && L.shared_gemm && L.Abf && groups == 1 && !g.a_idx && !g.c_idx && !g.grp_off && g.M >= 32 && g.N % 128 == 0 && g.K % 32 == 0 &&
+    if (bf && L.shared_gemm && L.Abf && groups == 1 && !g.a_idx && !g.c_idx && !g.grp_off && !g.mul && g.M >= 32 && g.N % 128 == 0 && g.K % 32 == 0 &&
         (!g.W2 || (g.ldc == g.N && L.G1 && L.G2))) {
         launch_lay_round_rows(g.A, g.lda, L.Abf, g.M, g.K, s);
         GemmArgs a{};
@@ -72,82 +80,162 @@ static void lay_gemm(Model& m, Layered& L, const LGemmArgs& g, int groups, hipSt
         if (ok && g.W2) { a.W = g.W2; a.C = L.G2; ok = launch_gemm(a, GEPI_STORE, s); }
         if (ok) {
             if (g.W2) launch_lay_act_mul(L.G1, L.G2, g.C, (size_t)g.M * g.N, g.act, s);
-            else launch_lay_act_cols(g.C, g.ldc, g.M, g.N, g.act, g.act2, g.act_split, s);
+            else launch_lay_act_cols(g.C, g.ldc, g.M, g.N, g.act, g.act2, g.act_split, s, g.act_param);
             return;
         }
     }
     launch_lgemm(g, bf, groups, s);
 }
 
-static int act_of(const std::string& s) { return s == "attention" ? LMIX_ATTN : (s == "lightning" ? LMIX_LIGHTNING : -1); }
+static void need(bool ok, const char* what) { if (!ok) throw CmError(CM_ERR_INVALID, std::string("config.json: ") + what); }
 
-// config.json of a layer-list decoder: "architecture", "vocab", "width", "residual_mult", "norm".eps, "canon".taps and "layers":
-// [{"type", "mixer": {...}, "mlp": null | {"kind": "dense", "ff"} | {"kind": "moe", "expert": {"ff"}, "router": {"experts", "top"}}}]
+// "mlp": null | {"kind": "dense", "ff"} | {"kind": "moe", "expert": {"ff"}, "router": {"experts", "top"}}
+static void parse_mlp(const cmjson::Value* ml, LayerSpec& sp, bool moe_ok) {
+    if (!ml || ml->kind != cmjson::Value::Obj) return;
+    const std::string kind = ml->string("kind", "dense");
+    if (kind == "dense") {
+        sp.mlp = LMLP_DENSE;
+        sp.ff = (int)ml->integer("ff", 0);
+    } else if (kind == "moe" && moe_ok) {
+        sp.mlp = LMLP_MOE;
+        const cmjson::Value* ex = ml->get("expert");
+        const cmjson::Value* rt = ml->get("router");
+        if (!ex || !rt) throw CmError(CM_ERR_IO, "config.json: moe without expert / router");
+        sp.ff = (int)ex->integer("ff", 0);
+        sp.experts = (int)rt->integer("experts", 0);
+        sp.top = (int)rt->integer("top", 0);
+        if (sp.experts <= 0 || sp.top <= 0 || sp.top > sp.experts || sp.experts > 4096) throw CmError(CM_ERR_INVALID, "router.experts / router.top");
+    } else throw CmError(CM_ERR_UNSUPPORTED, "mlp.kind '" + kind + "' not implemented");
+    if (sp.ff <= 0) throw CmError(CM_ERR_IO, "config.json: ff");
+}
+
+// Korupel: "residual_mult", "canon".taps; layer types "attention" (window + kept first tokens) and "lightning"
+static void parse_korupel_layer(const cmjson::Value& e, LayerSpec& sp) {
+    const std::string type = e.string("type", "");
+    sp.mixer = type == "attention" ? LMIX_ATTN : (type == "lightning" ? LMIX_LIGHTNING : -1);
+    if (sp.mixer < 0) throw CmError(CM_ERR_UNSUPPORTED, "layer type '" + type + "' not implemented");
+    const cmjson::Value* mx = e.get("mixer");
+    if (!mx || mx->kind != cmjson::Value::Obj) throw CmError(CM_ERR_IO, "config.json: layer without mixer");
+    sp.heads = (int)mx->integer("heads", 0);
+    sp.kv_heads = (int)mx->integer("kv_heads", sp.heads);
+    sp.dim = (int)mx->integer("dim", 0);
+    sp.vdim = (int)mx->integer("vdim", sp.dim);
+    if (sp.heads <= 0 || sp.dim <= 0 || sp.vdim <= 0) throw CmError(CM_ERR_IO, "config.json: mixer sizes");
+    if (sp.mixer == LMIX_ATTN) {
+        if (sp.kv_heads <= 0 || sp.heads % sp.kv_heads) throw CmError(CM_ERR_INVALID, "heads % kv_heads != 0");
+        if (sp.vdim != sp.dim) throw CmError(CM_ERR_INVALID, "attention whose values are its keys needs vdim == dim");
+        if (sp.dim > 256) throw CmError(CM_ERR_UNSUPPORTED, "attention head size above 256");
+        sp.scale = (float)mx->number("scale", 1.0 / std::sqrt((double)sp.dim));
+        sp.win = 1ll << 40; sp.keep = 0;
+        if (const cmjson::Value* mk = mx->get("mask"))
+            if (mk->kind == cmjson::Value::Obj) {
+                sp.win = mk->integer("size", sp.win);
+                sp.keep = mk->integer("keep_first", 0);
+            }
+        if (sp.win <= 0 || sp.keep < 0) throw CmError(CM_ERR_INVALID, "mask.size / mask.keep_first");
+        sp.bias = LBIAS_LOG; sp.gate = LGATE_HEAD;
+    } else {
+        if (sp.dim > 256) throw CmError(CM_ERR_UNSUPPORTED, "lightning head size above 256");
+        sp.kv_heads = sp.heads;
+        const cmjson::Value* dc = mx->get("decay");
+        if (dc && dc->kind == cmjson::Value::Arr) { for (auto& v : dc->arr) sp.decay.push_back((float)v->num); }
+        else sp.decay.assign((size_t)sp.heads, (float)mx->number("decay", 1.0));
+        if ((int)sp.decay.size() != sp.heads) throw CmError(CM_ERR_INVALID, "decay: one value per head");
+    }
+    parse_mlp(e.get("mlp"), sp, true);
+}
+
+// Mononex: layer types "attention" (position chunks, linear distance bias, sink, element-wise gate, optional "kv_from"),
+// "latent_attention" ("q_rank", "kv_rank", "rot_dim", "rot": {"base", "dims", "scaling": {"factor", "original", "fast", "slow"}})
+// and "gla" ("tau"); dense feed-forwards are W_down relu(W_up h)^2
+static void parse_mononex_layer(const cmjson::Value& e, LayerSpec& sp, const std::vector<LayerSpec>& before) {
+    const std::string type = e.string("type", "");
+    sp.mixer = type == "attention" ? LMIX_ATTN : (type == "latent_attention" ? LMIX_LATENT : (type == "gla" ? LMIX_GLA : -1));
+    if (sp.mixer < 0) throw CmError(CM_ERR_UNSUPPORTED, "layer type '" + type + "' not implemented");
+    const cmjson::Value* mx = e.get("mixer");
+    if (!mx || mx->kind != cmjson::Value::Obj) throw CmError(CM_ERR_IO, "config.json: layer without mixer");
+    sp.heads = (int)mx->integer("heads", 0);
+    sp.kv_heads = (int)mx->integer("kv_heads", sp.heads);
+    sp.dim = (int)mx->integer("dim", 0);
+    sp.vdim = (int)mx->integer("vdim", sp.dim);
+    need(sp.heads > 0 && sp.dim > 0 && sp.vdim > 0, "mixer sizes");
+    sp.win = 1ll << 40; sp.keep = 0;
+    if (sp.mixer == LMIX_ATTN) {
+        need(sp.kv_heads > 0 && sp.heads % sp.kv_heads == 0, "heads % kv_heads != 0");
+        sp.scale = (float)mx->number("scale", 1.0 / std::sqrt((double)sp.dim));
+        if (const cmjson::Value* mk = mx->get("mask"))
+            if (mk->kind == cmjson::Value::Obj) {
+                sp.chunk = mk->integer("size", 0);
+                need(sp.chunk > 0, "mask.size");
+            }
+        sp.bias = LBIAS_LINEAR; sp.gate = LGATE_ELEM; sp.sink = true; sp.own_v = true;
+        if (const cmjson::Value* kf = mx->get("kv_from"))
+            if (kf->kind == cmjson::Value::Num) {
+                sp.kv_from = (int)kf->num;
+                need(sp.kv_from >= 0 && sp.kv_from < (int)before.size(), "kv_from names no earlier layer");
+                const LayerSpec& src = before[(size_t)sp.kv_from];
+                need(src.mixer == LMIX_ATTN && src.kv_from < 0 && src.kv_heads == sp.kv_heads && src.dim == sp.dim && src.vdim == sp.vdim,
+                     "kv_from: the other layer's keys and values do not fit");
+            }
+        need(lay_attn_fits(sp.dim, sp.vdim, true), "attention head sizes too large");
+    } else if (sp.mixer == LMIX_LATENT) {
+        sp.q_rank = (int)mx->integer("q_rank", 0);
+        sp.kv_rank = (int)mx->integer("kv_rank", 0);
+        sp.rot_dim = (int)mx->integer("rot_dim", 0);
+        need(sp.q_rank > 0 && sp.kv_rank > 0 && sp.rot_dim >= 0, "q_rank / kv_rank / rot_dim");
+        sp.scale = (float)mx->number("scale", 1.0 / std::sqrt((double)(sp.dim + sp.rot_dim)));
+        sp.kv_heads = 1;               // one cached row per token: [latent | rotated key part]
+        sp.gate = LGATE_NONE;          // the gate acts on the values after their up-projection
+        if (const cmjson::Value* rt = mx->get("rot"))
+            if (rt->kind == cmjson::Value::Obj) {
+                sp.rot.dims = (int)rt->integer("dims", sp.rot_dim);
+                sp.rot.base = rt->number("base", 10000.0);
+                if (const cmjson::Value* sc = rt->get("scaling"))
+                    if (sc->kind == cmjson::Value::Obj) {
+                        sp.rot.yarn = true;
+                        sp.rot.factor = sc->number("factor", 1.0);
+                        sp.rot.original = sc->number("original", 0.0);
+                        sp.rot.fast = sc->number("fast", 32.0);
+                        sp.rot.slow = sc->number("slow", 1.0);
+                        need(sp.rot.factor > 0 && sp.rot.original > 0 && sp.rot.fast > 0 && sp.rot.slow > 0, "rot.scaling");
+                    }
+            }
+        need(sp.rot.dims >= 0 && sp.rot.dims <= sp.rot_dim && sp.rot.dims % 2 == 0 && sp.rot.base > 1.0, "rot.dims / rot.base");
+        need(lay_attn_fits(sp.kv_rank + sp.rot_dim, sp.kv_rank, false), "kv_rank + rot_dim too large");
+    } else {
+        sp.kv_heads = sp.heads;
+        sp.tau = (float)mx->number("tau", 1.0);
+        need(sp.tau > 0.f, "tau");
+        if (sp.dim > 256) throw CmError(CM_ERR_UNSUPPORTED, "gla head size above 256");
+    }
+    parse_mlp(e.get("mlp"), sp, false);
+    sp.gated_ff = false; sp.ff_act = LACT_RELU2;
+}
+
+// config.json of a layer-list decoder: "architecture", "vocab", "width", "norm".eps and "layers": [{"type", "mixer": {...}, "mlp"}]
 void Model::init_layered_config(const cmjson::Value& root) {
     const std::string arch = root.string("architecture", "");
-    if (arch != "Korupel") throw CmError(CM_ERR_UNSUPPORTED, "architecture '" + arch + "' not implemented (Korupel)");
+    if (arch != "Korupel" && arch != "Mononex") throw CmError(CM_ERR_UNSUPPORTED, "architecture '" + arch + "' not implemented (Korupel, Mononex)");
     layered = true;
     lay.reset(new Layered());
     Layered& L = *lay;
-    cfg.model_type = "korupel";
+    L.parallel = arch == "Mononex";
+    cfg.model_type = L.parallel ? "mononex" : "korupel";
     cfg.V = (int)root.integer("vocab", 0);
     cfg.H = (int)root.integer("width", 0);
     if (const cmjson::Value* n = root.get("norm")) cfg.eps = (float)n->number("eps", 1e-6);
-    if (const cmjson::Value* c = root.get("canon")) L.taps = (int)c->integer("taps", 0);
-    L.mult = (float)root.number("residual_mult", 1.0);
+    if (!L.parallel) {
+        if (const cmjson::Value* c = root.get("canon")) L.taps = (int)c->integer("taps", 0);
+        L.mult = (float)root.number("residual_mult", 1.0);
+    }
     const cmjson::Value* ls = root.get("layers");
     if (!ls || ls->kind != cmjson::Value::Arr || ls->arr.empty()) throw CmError(CM_ERR_IO, "config.json: no layers");
     if (cfg.V <= 0 || cfg.H <= 0) throw CmError(CM_ERR_IO, "config.json: vocab / width missing");
     if (L.taps < 0 || L.taps > 64) throw CmError(CM_ERR_UNSUPPORTED, "canon.taps out of range");
     for (auto& e : ls->arr) {
         LayerSpec sp;
-        sp.mixer = act_of(e->string("type", ""));
-        if (sp.mixer < 0) throw CmError(CM_ERR_UNSUPPORTED, "layer type '" + e->string("type", "") + "' not implemented");
-        const cmjson::Value* mx = e->get("mixer");
-        if (!mx || mx->kind != cmjson::Value::Obj) throw CmError(CM_ERR_IO, "config.json: layer without mixer");
-        sp.heads = (int)mx->integer("heads", 0);
-        sp.kv_heads = (int)mx->integer("kv_heads", sp.heads);
-        sp.dim = (int)mx->integer("dim", 0);
-        sp.vdim = (int)mx->integer("vdim", sp.dim);
-        if (sp.heads <= 0 || sp.dim <= 0 || sp.vdim <= 0) throw CmError(CM_ERR_IO, "config.json: mixer sizes");
-        if (sp.mixer == LMIX_ATTN) {
-            if (sp.kv_heads <= 0 || sp.heads % sp.kv_heads) throw CmError(CM_ERR_INVALID, "heads % kv_heads != 0");
-            if (sp.vdim != sp.dim) throw CmError(CM_ERR_INVALID, "attention whose values are its keys needs vdim == dim");
-            if (sp.dim > 256) throw CmError(CM_ERR_UNSUPPORTED, "attention head size above 256");
-            sp.scale = (float)mx->number("scale", 1.0 / std::sqrt((double)sp.dim));
-            sp.win = 1ll << 40; sp.keep = 0;
-            if (const cmjson::Value* mk = mx->get("mask"))
-                if (mk->kind == cmjson::Value::Obj) {
-                    sp.win = mk->integer("size", sp.win);
-                    sp.keep = mk->integer("keep_first", 0);
-                }
-            if (sp.win <= 0 || sp.keep < 0) throw CmError(CM_ERR_INVALID, "mask.size / mask.keep_first");
-        } else {
-            if (sp.dim > 256) throw CmError(CM_ERR_UNSUPPORTED, "lightning head size above 256");
-            sp.kv_heads = sp.heads;
-            const cmjson::Value* dc = mx->get("decay");
-            if (dc && dc->kind == cmjson::Value::Arr) { for (auto& v : dc->arr) sp.decay.push_back((float)v->num); }
-            else sp.decay.assign((size_t)sp.heads, (float)mx->number("decay", 1.0));
-            if ((int)sp.decay.size() != sp.heads) throw CmError(CM_ERR_INVALID, "decay: one value per head");
-        }
-        const cmjson::Value* ml = e->get("mlp");
-        if (ml && ml->kind == cmjson::Value::Obj) {
-            const std::string kind = ml->string("kind", "dense");
-            if (kind == "dense") {
-                sp.mlp = LMLP_DENSE;
-                sp.ff = (int)ml->integer("ff", 0);
-            } else if (kind == "moe") {
-                sp.mlp = LMLP_MOE;
-                const cmjson::Value* ex = ml->get("expert");
-                const cmjson::Value* rt = ml->get("router");
-                if (!ex || !rt) throw CmError(CM_ERR_IO, "config.json: moe without expert / router");
-                sp.ff = (int)ex->integer("ff", 0);
-                sp.experts = (int)rt->integer("experts", 0);
-                sp.top = (int)rt->integer("top", 0);
-                if (sp.experts <= 0 || sp.top <= 0 || sp.top > sp.experts || sp.experts > 4096) throw CmError(CM_ERR_INVALID, "router.experts / router.top");
-            } else throw CmError(CM_ERR_UNSUPPORTED, "mlp.kind '" + kind + "' not implemented");
-            if (sp.ff <= 0) throw CmError(CM_ERR_IO, "config.json: ff");
-        }
+        if (L.parallel) parse_mononex_layer(*e, sp, L.spec);
+        else parse_korupel_layer(*e, sp);
         L.spec.push_back(sp);
     }
     cfg.L = (int)L.spec.size();
@@ -170,6 +258,8 @@ struct LaySource {
     virtual ~LaySource() {}
     // values of tensor `name` with exactly n elements (bf16-representable for matrices)
     virtual std::vector<float> get(const std::string& name, size_t n, float synth_scale, float synth_off) = 0;
+    // first dimension of a tensor whose shape the configuration does not give (dflt: no checkpoint behind the source)
+    virtual int64_t dim0(const std::string& name, int64_t dflt) = 0;
 };
 
 struct LayFileSource : LaySource {
@@ -187,11 +277,17 @@ struct LayFileSource : LaySource {
         } else throw CmError(CM_ERR_UNSUPPORTED, "tensor " + name + ": dtype " + t.dtype);
         return out;
     }
+    int64_t dim0(const std::string& name, int64_t) override {
+        const cmst::TensorView& t = ck.get(name);
+        if (t.shape.empty()) throw CmError(CM_ERR_IO, "tensor " + name + ": unexpected shape");
+        return t.shape[0];
+    }
 };
 
 struct LaySynthSource : LaySource {
     uint64_t seed;
     explicit LaySynthSource(uint64_t s) : seed(s) {}
+    int64_t dim0(const std::string&, int64_t dflt) override { return dflt; }
     std::vector<float> get(const std::string& name, size_t n, float scale, float off) override {
         uint64_t h = 1469598103934665603ull ^ seed;
         for (char c : name) { h ^= (unsigned char)c; h *= 1099511628211ull; }
@@ -229,8 +325,36 @@ static uint16_t* up_bf16(Model& m, const std::vector<float>& v) {
 }
 static void append(std::vector<float>& dst, const std::vector<float>& src) { dst.insert(dst.end(), src.begin(), src.end()); }
 
+// angle per position of every rotated pair: base^(-2i / dims), with the YaRN blend between the original and the stretched
+// frequencies over the pair index, and the factor that goes on cos and sin
+static std::vector<float> rot_frequencies(const RotSpec& r, float* mag) {
+    const int half = r.dims / 2;
+    std::vector<float> f((size_t)half);
+    *mag = 1.f;
+    double lo = 0, hi = 0;
+    if (r.yarn) {
+        const double two_pi = 6.283185307179586476925286766559;
+        auto at = [&](double turns) { return r.dims * std::log(r.original / (two_pi * turns)) / (2.0 * std::log(r.base)); };
+        lo = std::max(std::floor(at(r.fast)), 0.0);
+        hi = std::min(std::ceil(at(r.slow)), (double)(r.dims - 1));
+        *mag = (float)(0.1 * std::log(r.factor) + 1.0);
+    }
+    for (int i = 0; i < half; ++i) {
+        double fi = std::pow(r.base, -2.0 * i / r.dims);
+        if (r.yarn) {
+            const double ramp = std::min(1.0, std::max(0.0, (i - lo) / std::max(hi - lo, 0.001)));
+            fi = fi / r.factor * ramp + fi * (1.0 - ramp);
+        }
+        f[(size_t)i] = (float)fi;
+    }
+    return f;
+}
+
+static void build_mononex(Model& m, LaySource& src);
+
 static void build_layered(Model& m, LaySource& src) {
     Layered& L = *m.lay;
+    if (L.parallel) { build_mononex(m, src); return; }
     const size_t W = (size_t)m.cfg.H, V = (size_t)m.cfg.V;
     const float ws = 1.0f / std::sqrt((float)W);
     m.embed = up_bf16(m, src.get("embed", V * W, 1.0f, 0.f));
@@ -298,6 +422,95 @@ static void build_layered(Model& m, LaySource& src) {
     m.lm_head = L.head;
 }
 
+// norm weights stored around zero: the factor is 1 + w
+static std::vector<float> plus_one(std::vector<float> v) { for (float& x : v) x += 1.f; return v; }
+
+static void build_mononex(Model& m, LaySource& src) {
+    Layered& L = *m.lay;
+    const size_t W = (size_t)m.cfg.H, V = (size_t)m.cfg.V;
+    const float ws = 1.0f / std::sqrt((float)W);
+    m.embed = up_bf16(m, src.get("embed", V * W, 1.0f, 0.f));
+    L.w.resize(L.spec.size());
+    int kv_idx = 0;
+    for (size_t i = 0; i < L.spec.size(); ++i) {
+        LayerSpec& sp = L.spec[i];
+        LayeredLayerW& w = L.w[i];
+        const std::string p = "l" + std::to_string(i) + ".";
+        w.norm1 = up_f32(m, plus_one(src.get(p + "norm1", W, 0.1f, 0.f)));
+        {   // token shift h + (h' - h) s as the two-tap convolution h + s h' - s h
+            const std::vector<float> sh = src.get(p + "shift", W, 0.25f, 0.5f);
+            std::vector<float> cw(2 * W);
+            for (size_t c = 0; c < W; ++c) { cw[2 * c] = sh[c]; cw[2 * c + 1] = -sh[c]; }
+            w.shift = up_f32(m, cw);
+        }
+        const size_t H = (size_t)sp.heads, G = (size_t)sp.kv_heads, d = (size_t)sp.dim, e = (size_t)sp.vdim;
+        std::vector<float> in;
+        if (sp.mixer == LMIX_ATTN) {
+            const bool own = sp.kv_from < 0;
+            w.q_off = 0; w.k_off = (int)(H * d); w.v_off = w.k_off + (own ? (int)(G * d) : 0); w.g_off = w.v_off + (own ? (int)(G * e) : 0);
+            w.in_rows = w.g_off + (int)(H * e);
+            append(in, src.get(p + "mix.q", H * d * W, ws, 0.f));
+            if (own) {
+                append(in, src.get(p + "mix.k", G * d * W, ws, 0.f));
+                append(in, src.get(p + "mix.v", G * e * W, ws, 0.f));
+            }
+            append(in, src.get(p + "mix.g", H * e * W, ws, 0.f));
+            w.sink = up_f32(m, src.get(p + "mix.sink", H, 1.0f, 0.f));
+            std::vector<float> slope(H);
+            for (size_t h = 0; h < H; ++h) slope[h] = (float)std::pow(2.0, -8.0 * (double)(h + 1) / (double)H);
+            w.r1 = up_f32(m, slope);
+            w.o_w = up_bf16(m, src.get(p + "mix.o", W * H * e, 1.0f / std::sqrt((float)(H * e)), 0.f));
+            w.kv_idx = kv_idx++;
+        } else if (sp.mixer == LMIX_LATENT) {
+            const size_t qr = (size_t)sp.q_rank, kr = (size_t)sp.kv_rank, r = (size_t)sp.rot_dim;
+            w.q_off = 0; w.k_off = (int)qr; w.g_off = (int)(qr + kr + r); w.in_rows = w.g_off + (int)(H * e);
+            append(in, src.get(p + "mix.dq", qr * W, ws, 0.f));
+            append(in, src.get(p + "mix.dkv", (kr + r) * W, ws, 0.f));
+            append(in, src.get(p + "mix.g", H * e * W, ws, 0.f));
+            w.dq_norm = up_f32(m, src.get(p + "mix.dq.norm", qr, 0.1f, 1.f));
+            w.dkv_norm = up_f32(m, src.get(p + "mix.dkv.norm", kr, 0.1f, 1.f));
+            w.uq = up_bf16(m, src.get(p + "mix.uq", H * (d + r) * qr, 1.0f / std::sqrt((float)qr), 0.f));
+            {   // W_uk per head, transposed: the product q_unrotated . (W_uk c) = (W_uk^T q_unrotated) . c runs against the cached latent
+                const std::vector<float> uk = src.get(p + "mix.uk", H * d * kr, 1.0f / std::sqrt((float)kr), 0.f);
+                std::vector<float> t(H * kr * d);
+                for (size_t h = 0; h < H; ++h)
+                    for (size_t a = 0; a < d; ++a)
+                        for (size_t c = 0; c < kr; ++c) t[(h * kr + c) * d + a] = uk[(h * d + a) * kr + c];
+                w.uk_t = up_bf16(m, t);
+            }
+            w.uv = up_bf16(m, src.get(p + "mix.uv", H * e * kr, 1.0f / std::sqrt((float)kr), 0.f));
+            if (sp.rot.dims > 0) w.rot_freq = up_f32(m, rot_frequencies(sp.rot, &w.rot_mag));
+            w.o_w = up_bf16(m, src.get(p + "mix.o", W * H * e, 1.0f / std::sqrt((float)(H * e)), 0.f));
+            w.kv_idx = kv_idx++;
+        } else {
+            sp.a_rank = (int)src.dim0(p + "mix.a1", 16);
+            if (sp.a_rank <= 0) throw CmError(CM_ERR_IO, "tensor " + p + "mix.a1: unexpected shape");
+            const size_t ar = (size_t)sp.a_rank;
+            w.q_off = 0; w.k_off = (int)(H * d); w.v_off = (int)(2 * H * d); w.a_off = (int)(2 * H * d + H * e);
+            w.g_off = w.a_off + (int)ar; w.in_rows = w.g_off + (int)(H * e);
+            append(in, src.get(p + "mix.q", H * d * W, ws, 0.f));
+            append(in, src.get(p + "mix.k", H * d * W, ws, 0.f));
+            append(in, src.get(p + "mix.v", H * e * W, ws, 0.f));
+            append(in, src.get(p + "mix.a1", ar * W, ws, 0.f));
+            append(in, src.get(p + "mix.g", H * e * W, ws, 0.f));
+            w.a2 = up_bf16(m, src.get(p + "mix.a2", H * d * ar, 1.0f / std::sqrt((float)ar), 0.f));
+            w.a2_b = up_f32(m, src.get(p + "mix.a2.b", H * d, 1.0f, 2.f));
+            w.mix_norm = up_f32(m, src.get(p + "mix.norm", e, 0.1f, 1.f));
+            w.o_w = up_bf16(m, src.get(p + "mix.o", W * H * e, 1.0f / std::sqrt((float)(H * e)), 0.f));
+        }
+        w.in_w = up_bf16(m, in);
+        if (sp.mlp != LMLP_NONE) {
+            w.norm2 = up_f32(m, plus_one(src.get(p + "norm2", W, 0.1f, 0.f)));
+            const size_t ff = (size_t)sp.ff;
+            w.up = up_bf16(m, src.get(p + "mlp.up", ff * W, ws, 0.f));
+            w.down = up_bf16(m, src.get(p + "mlp.down", W * ff, 1.0f / std::sqrt((float)ff), 0.f));
+        }
+    }
+    L.final_norm = up_f32(m, plus_one(src.get("final.norm", W, 0.1f, 0.f)));
+    L.head = up_bf16(m, src.get("head", V * W, ws, 0.f));
+    m.lm_head = L.head;
+}
+
 void load_layered_from_dir(Model& m, const std::string& dir) {
     try {
         LayFileSource src(dir);
@@ -327,24 +540,51 @@ void Model::alloc_runtime_layered() {
     for (size_t i = 0; i < L.spec.size(); ++i) {
         const LayerSpec& sp = L.spec[i];
         LayeredLayerW& w = L.w[i];
-        if (sp.mixer == LMIX_ATTN) {
-            kv_index[i] = n_kv_layers++;
-            w.k_page_bytes = (size_t)sp.kv_heads * page * sp.dim * kv_esize;
-            w.k_pool_off = pool_bytes;
-            pool_bytes += (size_t)n_pages * w.k_page_bytes;
-            page_bytes += w.k_page_bytes;      // all layers' share of one page (kv_bytes)
+        if (sp.mixer == LMIX_ATTN || sp.mixer == LMIX_LATENT) {
+            // cached row of a token and key head: the key (latent attention: [latent | rotated key part], one head); values that
+            // are not (a part of) the keys have pages of their own
+            const int dk = sp.mixer == LMIX_LATENT ? sp.kv_rank + sp.rot_dim : sp.dim;
+            const int ev = sp.mixer == LMIX_LATENT ? sp.kv_rank : sp.vdim;
+            if (sp.kv_from >= 0) {             // the other layer's pages
+                const LayeredLayerW& o = L.w[(size_t)sp.kv_from];
+                w.k_pool_off = o.k_pool_off; w.k_page_bytes = o.k_page_bytes; w.v_pool_off = o.v_pool_off; w.v_page_bytes = o.v_page_bytes;
+                w.kv_idx = -1;
+            } else {
+                kv_index[i] = n_kv_layers++;
+                w.k_page_bytes = (size_t)sp.kv_heads * page * dk * kv_esize;
+                w.k_pool_off = pool_bytes;
+                pool_bytes += (size_t)n_pages * w.k_page_bytes;
+                page_bytes += w.k_page_bytes;      // all layers' share of one page (kv_bytes)
+                if (sp.own_v) {
+                    pool_bytes = (pool_bytes + 15) / 16 * 16;
+                    w.v_page_bytes = (size_t)sp.kv_heads * page * sp.vdim * kv_esize;
+                    w.v_pool_off = pool_bytes;
+                    pool_bytes += (size_t)n_pages * w.v_page_bytes;
+                    page_bytes += w.v_page_bytes;
+                }
+                pool_bytes = (pool_bytes + 15) / 16 * 16;
+            }
             const int nrep = sp.heads / sp.kv_heads;
             if (std::find(L.nreps.begin(), L.nreps.end(), nrep) == L.nreps.end()) L.nreps.push_back(nrep);
-            L.max_o = std::max(L.max_o, sp.heads * sp.dim);
+            L.max_o = std::max(L.max_o, sp.heads * ev);
+            L.max_e = std::max(L.max_e, ev);
+            if (sp.mixer == LMIX_LATENT) {
+                L.max_o = std::max(L.max_o, sp.heads * sp.vdim);
+                L.max_cq = std::max(L.max_cq, sp.q_rank);
+                L.max_q = std::max(L.max_q, sp.heads * (sp.dim + sp.rot_dim));
+                L.max_qa = std::max(L.max_qa, sp.heads * dk);
+            }
         } else {
             w.st_off = st;
             st += (size_t)sp.heads * sp.dim * sp.vdim;
             L.max_o = std::max(L.max_o, sp.heads * sp.vdim);
+            if (sp.mixer == LMIX_GLA) L.max_ld = std::max(L.max_ld, sp.heads * sp.dim);
         }
         if (L.taps > 1) {
             w.c1_off = cv; cv += (size_t)(L.taps - 1) * W;
             if (sp.mlp != LMLP_NONE) { w.c2_off = cv; cv += (size_t)(L.taps - 1) * W; }
         }
+        if (w.shift) { w.sh_off = cv; cv += W; }       // the mixer's previous input
         L.max_in = std::max(L.max_in, w.in_rows);
         if (sp.mlp != LMLP_NONE) L.max_ff = std::max(L.max_ff, sp.ff);
         if (sp.mlp == LMLP_MOE) { L.max_top = std::max(L.max_top, sp.top); L.max_E = std::max(L.max_E, sp.experts); }
@@ -376,6 +616,13 @@ void Model::alloc_runtime_layered() {
     L.O = dalloc<float>(cap * (size_t)L.max_o);
     L.O2 = dalloc<float>(cap * (size_t)L.max_o);
     if (L.max_ff) L.HH = dalloc<float>(cap * (size_t)L.max_top * (size_t)L.max_ff);
+    if (L.parallel) { L.H2 = dalloc<float>(cap * W); L.Y2 = dalloc<float>(cap * W); }
+    if (L.max_cq) {
+        L.CQ = dalloc<float>(cap * (size_t)L.max_cq);
+        L.Q = dalloc<float>(cap * (size_t)L.max_q);
+        L.Qa = dalloc<float>(cap * (size_t)L.max_qa);
+    }
+    if (L.max_ld) L.LD = dalloc<float>(cap * (size_t)L.max_ld);
     if (L.max_E > 1 || L.max_top > 1 || std::any_of(L.spec.begin(), L.spec.end(), [](const LayerSpec& s) { return s.mlp == LMLP_MOE; })) {
         L.YS = dalloc<float>(cap * (size_t)L.max_top * W);
         L.wsel = dalloc<float>(cap * (size_t)L.max_top);
@@ -384,22 +631,23 @@ void Model::alloc_runtime_layered() {
         L.off = dalloc<int32_t>((size_t)L.max_E + 1);
     }
     if (!L.f32) {
-        int max_k = std::max((int)W, std::max(L.max_o, L.max_ff)), dense_ff = 0;
-        for (const LayerSpec& sp : L.spec) if (sp.mlp == LMLP_DENSE) dense_ff = std::max(dense_ff, sp.ff);
+        int max_k = std::max({(int)W, L.max_o, L.max_ff, L.max_cq}), dense_ff = 0;
+        for (const LayerSpec& sp : L.spec) if (sp.mlp == LMLP_DENSE && sp.gated_ff) dense_ff = std::max(dense_ff, sp.ff);
         const size_t rows = (cap + 255) / 256 * 256;
         L.Abf = dalloc<uint16_t>(rows * (size_t)max_k);
         CM_HIP(hipMemsetAsync(L.Abf, 0, rows * (size_t)max_k * sizeof(uint16_t), stream));
         if (dense_ff) { L.G1 = dalloc<float>(cap * (size_t)dense_ff); L.G2 = dalloc<float>(cap * (size_t)dense_ff); }
         ensure_gemm_workspace();
     }
-    size_t hde = 0; int max_d = 0;
+    size_t hde = 0, hd = 0;
     for (const LayerSpec& sp : L.spec) {
-        if (sp.mixer == LMIX_LIGHTNING && sp.dim <= 128) hde = std::max(hde, (size_t)sp.heads * sp.dim * sp.vdim);
-        if (sp.mixer == LMIX_ATTN) max_d = std::max(max_d, sp.dim);
+        if ((sp.mixer == LMIX_LIGHTNING || sp.mixer == LMIX_GLA) && sp.dim <= 128) hde = std::max(hde, (size_t)sp.heads * sp.dim * sp.vdim);
+        if (sp.mixer == LMIX_GLA && sp.dim <= 128) hd = std::max(hd, (size_t)sp.heads * sp.dim);
     }
     if (hde) { L.u_stride = hde; L.U = dalloc<float>((cap / LAY_LIGHT_CHUNK + (size_t)MAXB + 1) * hde); }
-    if (max_d) {
-        L.att_po = dalloc<float>((size_t)Layered::ATT_PARTS * 16 * max_d);
+    if (hd) L.Dch = dalloc<float>((cap / LAY_LIGHT_CHUNK + (size_t)MAXB + 1) * hd);
+    if (L.max_e) {
+        L.att_po = dalloc<float>((size_t)Layered::ATT_PARTS * 16 * L.max_e);
         L.att_pml = dalloc<float>((size_t)Layered::ATT_PARTS * 16 * 2);
     }
     L.am_pv = dalloc<float>((size_t)Layered::LOGIT_ROWS * LAY_ARGMAX_PARTS);
@@ -448,6 +696,9 @@ void Model::layered_cow_page(int32_t oldp, int32_t newp) {
         if (w.kv_idx < 0) continue;
         CM_HIP(hipMemcpyAsync(kv_pool + w.k_pool_off + (size_t)newp * w.k_page_bytes, kv_pool + w.k_pool_off + (size_t)oldp * w.k_page_bytes,
                               w.k_page_bytes, hipMemcpyDeviceToDevice, stream));
+        if (w.v_page_bytes)
+            CM_HIP(hipMemcpyAsync(kv_pool + w.v_pool_off + (size_t)newp * w.v_page_bytes, kv_pool + w.v_pool_off + (size_t)oldp * w.v_page_bytes,
+                                  w.v_page_bytes, hipMemcpyDeviceToDevice, stream));
     }
 }
 
@@ -593,9 +844,131 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             launch_lay_canon(L.Hn, L.Hc, cw, conv_pool, conv_slot_elems, coff, d_segs, d_rowseg, T, W, L.taps, s);
             launch_lay_canon_tail(L.Hn, conv_pool, conv_slot_elems, coff, d_segs, nseg, W, L.taps, s);
         };
+        // softmax attention of one layer over the pages: queries at qsrc[row ldq + q_off + head dk], output [T][H ev] into L.O
+        auto run_attention = [&](const LayerSpec& sp, const LayeredLayerW& w, const float* qsrc, int ldq, int q_off, int g_off, int dk, int ev) {
+            LAttnArgs a;
+            a.proj = qsrc; a.ldp = ldq; a.q_off = q_off; a.g_off = g_off;
+            a.out = L.O; a.ldo = sp.heads * ev;
+            a.kpool = kv_pool + w.k_pool_off; a.bt = d_bt; a.segs = d_segs;
+            a.vpool = w.v_page_bytes ? kv_pool + w.v_pool_off : nullptr; a.e = ev;
+            const auto& tl = tiles[sp.heads / sp.kv_heads];
+            a.tiles = (const int2*)(L.d_tab + tl.first); a.ntiles = tl.second;
+            a.r1 = w.r1; a.r2 = w.r2; a.H = sp.heads; a.G = sp.kv_heads; a.d = dk; a.page = page;
+            a.scale = sp.scale; a.win = sp.win; a.keep = sp.keep; a.chunk = sp.chunk;
+            a.bias = sp.bias; a.gate = sp.gate; a.sink = sp.sink ? w.sink : nullptr;
+            {   // few query tiles and many visible keys (decode steps): share a tile's keys among blocks
+                long long seen = std::min<long long>(max_len, sp.win + sp.keep);
+                if (sp.chunk > 0) seen = std::min(seen, sp.chunk);
+                const int key_tiles = (int)((seen + 63) / 64), blocks = std::max(1, a.ntiles * sp.kv_heads);
+                a.nsplit = std::max(1, std::min({32, key_tiles, 256 / blocks, Layered::ATT_PARTS / blocks}));
+                a.part_o = L.att_po; a.part_ml = L.att_pml;
+            }
+            const bool plain = sp.bias == LBIAS_LOG && sp.gate == LGATE_HEAD && !sp.sink && sp.chunk == 0 && !a.vpool && ev == dk;
+            if (plain && L.attn_mfma && kv_mode == KV_BF16 && !all_decode && max_n >= 16 && dk % 16 == 0 && dk <= 128) {
+                const auto& tm = tiles64[sp.heads / sp.kv_heads];
+                a.tiles = (const int2*)(L.d_tab + tm.first); a.ntiles = tm.second;
+                launch_lay_attn_mfma(a, s);
+            } else
+                launch_lay_attn(a, kv_mode, s);
+        };
+        // lightning / gated linear attention of one layer: raw head outputs into L.O
+        auto run_linear = [&](const LayerSpec& sp, const LayeredLayerW& w, const float* ldec) {
+            LLightArgs a;
+            a.proj = L.P; a.ldp = w.in_rows; a.q_off = w.q_off; a.k_off = w.k_off; a.v_off = w.v_off;
+            a.out = L.O; a.ldo = sp.heads * sp.vdim;
+            a.state_pool = state_pool; a.slot_stride = state_slot_elems; a.st_off = w.st_off;
+            a.segs = d_segs; a.nseg = nseg; a.decay = w.decay; a.H = sp.heads; a.d = sp.dim; a.e = sp.vdim;
+            a.all_single = all_decode;
+            if (ldec) { a.ldec = ldec; a.ldd = sp.heads * sp.dim; a.qscale = 1.0f / std::sqrt((float)sp.dim); a.D = L.Dch; }
+            if (L.U && max_n > LAY_LIGHT_CHUNK && sp.dim <= 128) {       // a long portion in the pass: parallel over chunks
+                a.U = L.U; a.chunks = (const int2*)(L.d_tab + o_chunks); a.nchunks = nchunks;
+            }
+            launch_lay_lightning(a, s);
+        };
+        const float *par_y1 = nullptr, *par_y2 = nullptr;       // parallel layers: sublayer outputs not yet added to the residual
         for (size_t li = 0; li < L.spec.size(); ++li) {
             const LayerSpec& sp = L.spec[li];
             const LayeredLayerW& w = L.w[li];
+            if (L.parallel) {
+                // ---- mixer and feed-forward side by side on two norms of the same residual; the mixer's rows pass the token shift
+                float* h2 = sp.mlp != LMLP_NONE ? L.H2 : nullptr;
+                if (all_decode) {          // one launch: the previous layer's residual update, both norms, the shift and its state
+                    launch_lay_add_norm2_shift_decode(L.X, par_y1, par_y2, w.norm1, w.norm2, cfg.eps, L.Hc, h2, w.shift, conv_pool, conv_slot_elems,
+                                                      w.sh_off, d_segs, T, W, s);
+                    par_y1 = par_y2 = nullptr;
+                } else {
+                    launch_lay_rms_rows2(L.X, w.norm1, w.norm2, L.Hn, h2, T, W, cfg.eps, s);
+                    launch_lay_canon(L.Hn, L.Hc, w.shift, conv_pool, conv_slot_elems, w.sh_off, d_segs, d_rowseg, T, W, 2, s);
+                    launch_lay_canon_tail(L.Hn, conv_pool, conv_slot_elems, w.sh_off, d_segs, nseg, W, 2, s);
+                }
+                LGemmArgs g;
+                g.A = L.Hc; g.lda = W; g.W = w.in_w; g.C = L.P; g.ldc = w.in_rows; g.M = T; g.N = w.in_rows; g.K = W;
+                g.act_split = w.g_off; g.act = LACT_NONE; g.act2 = sp.mixer == LMIX_GLA ? LACT_SILU : LACT_SIGMOID;
+                lay_gemm(*this, L, g, 1, s);
+                const int H = sp.heads, ev = sp.vdim;
+                const float* oa = L.O;
+                if (sp.mixer == LMIX_ATTN) {
+                    if (sp.kv_from < 0) {
+                        launch_lay_k_append(L.P, w.in_rows, w.k_off, kv_pool + w.k_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, sp.kv_heads, sp.dim, page, s);
+                        launch_lay_k_append(L.P, w.in_rows, w.v_off, kv_pool + w.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, sp.kv_heads, ev, page, s);
+                    }
+                    run_attention(sp, w, L.P, w.in_rows, w.q_off, w.g_off, sp.dim, ev);
+                } else if (sp.mixer == LMIX_LATENT) {
+                    const int kr = sp.kv_rank, r = sp.rot_dim, dh = sp.dim, dk = kr + r;
+                    // both latents through their norms; the key latent in place, next to the shared rotated key part
+                    launch_lay_rms_cols(L.P, w.in_rows, w.q_off, sp.q_rank, w.dq_norm, L.CQ, sp.q_rank, T, cfg.eps, s);
+                    launch_lay_rms_cols(L.P, w.in_rows, w.k_off, kr, w.dkv_norm, L.P + w.k_off, w.in_rows, T, cfg.eps, s);
+                    LGemmArgs gq;
+                    gq.A = L.CQ; gq.lda = sp.q_rank; gq.W = w.uq; gq.C = L.Q; gq.ldc = H * (dh + r); gq.M = T; gq.N = H * (dh + r); gq.K = sp.q_rank;
+                    lay_gemm(*this, L, gq, 1, s);
+                    if (r > 0 && sp.rot.dims > 0)
+                        launch_lay_rope(L.P + w.k_off + kr, w.in_rows, 0, L.P + w.k_off + kr, w.in_rows, 0, 1, r, sp.rot.dims, w.rot_freq, w.rot_mag,
+                                        d_segs, d_rowseg, T, s);
+                    launch_lay_k_append(L.P, w.in_rows, w.k_off, kv_pool + w.k_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, 1, dk, page, s);
+                    // q_unrotated . (W_uk c) = (W_uk^T q_unrotated) . c: per head, the query moves into the latent's space
+                    LGemmArgs ga;
+                    ga.A = L.Q; ga.lda = H * (dh + r); ga.a_goff = (size_t)(dh + r); ga.W = w.uk_t; ga.w_stride = (size_t)kr * dh;
+                    ga.C = L.Qa; ga.ldc = H * dk; ga.c_goff = (size_t)dk; ga.M = T; ga.N = kr; ga.K = dh;
+                    lay_gemm(*this, L, ga, H, s);
+                    if (r > 0)
+                        launch_lay_rope(L.Q + dh, H * (dh + r), dh + r, L.Qa + kr, H * dk, dk, H, r, sp.rot.dims, w.rot_freq, w.rot_mag, d_segs,
+                                        d_rowseg, T, s);
+                    run_attention(sp, w, L.Qa, H * dk, 0, 0, dk, kr);
+                    // the weighted latents become values per head, times the gate
+                    LGemmArgs gv;
+                    gv.A = L.O; gv.lda = H * kr; gv.a_goff = (size_t)kr; gv.W = w.uv; gv.w_stride = (size_t)ev * kr;
+                    gv.C = L.O2; gv.ldc = H * ev; gv.c_goff = (size_t)ev; gv.M = T; gv.N = ev; gv.K = kr;
+                    gv.mul = L.P + w.g_off; gv.ldm = w.in_rows;
+                    lay_gemm(*this, L, gv, H, s);
+                    oa = L.O2;
+                } else {
+                    // logarithm of the decay: ln(sigmoid(z)^(1 / tau)), z from the low-rank pair
+                    LGemmArgs gd;
+                    gd.A = L.P + w.a_off; gd.lda = w.in_rows; gd.W = w.a2; gd.bias = w.a2_b; gd.C = L.LD; gd.ldc = H * sp.dim;
+                    gd.M = T; gd.N = H * sp.dim; gd.K = sp.a_rank; gd.act = LACT_LOGSIG; gd.act_split = gd.N; gd.act_param = 1.0f / sp.tau;
+                    lay_gemm(*this, L, gd, 1, s);
+                    run_linear(sp, w, L.LD);
+                    launch_lay_rms_gate(L.O, L.P + w.g_off, w.in_rows, w.mix_norm, L.O2, T, H * ev, cfg.eps, s, ev, true);
+                    oa = L.O2;
+                }
+                LGemmArgs go;
+                go.A = oa; go.lda = H * ev; go.W = w.o_w; go.C = L.Y; go.ldc = W; go.M = T; go.N = W; go.K = H * ev;
+                lay_gemm(*this, L, go, 1, s);
+                if (sp.mlp != LMLP_NONE) {
+                    LGemmArgs gu;
+                    gu.A = L.H2; gu.lda = W; gu.W = w.up; gu.C = L.HH; gu.ldc = sp.ff; gu.M = T; gu.N = sp.ff; gu.K = W;
+                    gu.act = sp.ff_act; gu.act_split = sp.ff;
+                    lay_gemm(*this, L, gu, 1, s);
+                    LGemmArgs dn;
+                    dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.C = L.Y2; dn.ldc = W; dn.M = T; dn.N = W; dn.K = sp.ff;
+                    lay_gemm(*this, L, dn, 1, s);
+                }
+                par_y1 = L.Y; par_y2 = sp.mlp != LMLP_NONE ? L.Y2 : nullptr;
+                if (!all_decode || L.capture || li + 1 == L.spec.size()) {      // decode steps: inside the next layer's first launch
+                    launch_lay_add_rows(L.X, par_y1, par_y2, (size_t)T * W, s);
+                    par_y1 = par_y2 = nullptr;
+                }
+            } else {
             norm_canon(w.norm1, w.canon1, w.c1_off);
             LGemmArgs g;
             g.A = L.Hc; g.lda = W; g.W = w.in_w; g.bias = w.in_b; g.C = L.P; g.ldc = w.in_rows; g.M = T; g.N = w.in_rows; g.K = W;
@@ -605,40 +978,11 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             int on = 0;
             const float* oa = nullptr;
             if (sp.mixer == LMIX_ATTN) {
-                void* kp = kv_pool + w.k_pool_off;
-                launch_lay_k_append(L.P, w.in_rows, w.k_off, kp, kv_mode, d_bt, d_segs, d_rowseg, T, sp.kv_heads, sp.dim, page, s);
-                LAttnArgs a;
-                a.proj = L.P; a.ldp = w.in_rows; a.q_off = w.q_off; a.g_off = w.g_off;
-                a.out = L.O; a.ldo = sp.heads * sp.dim;
-                a.kpool = kp; a.bt = d_bt; a.segs = d_segs;
-                const auto& tl = tiles[sp.heads / sp.kv_heads];
-                a.tiles = (const int2*)(L.d_tab + tl.first); a.ntiles = tl.second;
-                a.r1 = w.r1; a.r2 = w.r2; a.H = sp.heads; a.G = sp.kv_heads; a.d = sp.dim; a.page = page;
-                a.scale = sp.scale; a.win = sp.win; a.keep = sp.keep;
-                {   // few query tiles and many visible keys (decode steps): share a tile's keys among blocks
-                    const long long seen = std::min<long long>(max_len, sp.win + sp.keep);
-                    const int key_tiles = (int)((seen + 63) / 64), blocks = std::max(1, a.ntiles * sp.kv_heads);
-                    a.nsplit = std::max(1, std::min({32, key_tiles, 256 / blocks, Layered::ATT_PARTS / blocks}));
-                    a.part_o = L.att_po; a.part_ml = L.att_pml;
-                }
-                if (L.attn_mfma && kv_mode == KV_BF16 && !all_decode && max_n >= 16 && sp.dim % 16 == 0 && sp.dim <= 128) {
-                    const auto& tm = tiles64[sp.heads / sp.kv_heads];
-                    a.tiles = (const int2*)(L.d_tab + tm.first); a.ntiles = tm.second;
-                    launch_lay_attn_mfma(a, s);
-                } else
-                launch_lay_attn(a, kv_mode, s);
+                launch_lay_k_append(L.P, w.in_rows, w.k_off, kv_pool + w.k_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, sp.kv_heads, sp.dim, page, s);
+                run_attention(sp, w, L.P, w.in_rows, w.q_off, w.g_off, sp.dim, sp.dim);
                 on = sp.heads * sp.dim; oa = L.O;
             } else {
-                LLightArgs a;
-                a.proj = L.P; a.ldp = w.in_rows; a.q_off = w.q_off; a.k_off = w.k_off; a.v_off = w.v_off;
-                a.out = L.O; a.ldo = sp.heads * sp.vdim;
-                a.state_pool = state_pool; a.slot_stride = state_slot_elems; a.st_off = w.st_off;
-                a.segs = d_segs; a.nseg = nseg; a.decay = w.decay; a.H = sp.heads; a.d = sp.dim; a.e = sp.vdim;
-                a.all_single = all_decode;
-                if (L.U && max_n > LAY_LIGHT_CHUNK && sp.dim <= 128) {       // a long portion in the pass: parallel over chunks
-                    a.U = L.U; a.chunks = (const int2*)(L.d_tab + o_chunks); a.nchunks = nchunks;
-                }
-                launch_lay_lightning(a, s);
+                run_linear(sp, w, nullptr);
                 on = sp.heads * sp.vdim;
                 launch_lay_rms_gate(L.O, L.P + w.g_off, w.in_rows, w.mix_norm, L.O2, T, on, cfg.eps, s);
                 oa = L.O2;
@@ -672,6 +1016,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     lay_gemm(*this, L, dn, sp.experts, s);
                     post_norm(L.YS, w.norm2b, L.wsel, sp.top);
                 }
+            }
             }
             if (L.capture || li + 1 == L.spec.size()) flush_post();
             if (L.capture) {
