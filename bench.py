@@ -145,11 +145,11 @@ def relaunch_under_torchrun(n: int) -> int:
     return subprocess.call(cmd, env=env)
 
 
-def korupel_leg(args):
-    """--korupel: prompt and decode throughput of the Korupel decoder (layer-list family, crane_amd/csrc/model_layered.cpp) at the
-    widths of a real model, random weights, beside the closest family of the library at equal size: the Qwen3.5 hybrid (linear
-    attention 3 : 1 softmax attention, same width / ff / layers / vocabulary).  One JSON line; the default workload of this script
-    is not touched."""
+def korupel_leg(args, names=None, prompt_lens=None, label="korupel"):
+    """--korupel / --mononex: prompt and decode throughput of a layer-list decoder (Korupel, Mononex; crane_amd/csrc/model_layered.cpp)
+    at the widths of a real model, random weights, beside the closest family of the library at equal size: the Qwen3.5 hybrid
+    (linear attention 3 : 1 softmax attention, same width / ff / layers / vocabulary).  One JSON line; the default workload of this
+    script is not touched."""
     import numpy as np
     from crane_amd import configs
     from crane_amd.backend import Model
@@ -162,10 +162,10 @@ def korupel_leg(args):
 
     rows = []
     ctx, K = args.ctx, args.steps
-    prompts = [int(x) for x in args.korupel_prompts.split(",")]
-    for name in args.korupel.split(","):
+    prompts = [int(x) for x in (prompt_lens or args.korupel_prompts).split(",")]
+    for name in (names or args.korupel).split(","):
         cfg = configs.get_config(name)
-        lay = cfg.get("architecture") == "Korupel"
+        lay = "architecture" in cfg and "layers" in cfg
         V = cfg["vocab"] if lay else cfg["vocab_size"]
         m = Model.synthetic(cfg, seed=0, max_seq_len=max(4096, ctx + K + 64), max_seqs=34, kv_dtype="bf16",
                             prefill_split=1, **({"compute_dtype": "bfloat16"} if lay else {}))
@@ -209,7 +209,7 @@ def korupel_leg(args):
         r["decode"]["32"] = {"ms_per_round": round(dt * 1e3, 3), "tok_s": round(B / dt, 1)}
         m.close()
         rows.append(r)
-    print(json.dumps({"metric": "korupel prompt / decode throughput beside the closest family at equal size", "unit": "tokens/s",
+    print(json.dumps({"metric": label + " prompt / decode throughput beside the closest family at equal size", "unit": "tokens/s",
                       "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}))
     return 0
 
@@ -247,9 +247,14 @@ def main():
     ap.add_argument("--korupel", default=None, metavar="CONFIGS", help="comma-separated registry configs (e.g. korupel-1b,qwen3.5-0.8b): "
                     "prompt and decode throughput of each instead of the headline workload")
     ap.add_argument("--korupel-prompts", default="512,2048", help="prompt lengths of --korupel")
+    ap.add_argument("--mononex", default=None, metavar="CONFIGS", help="comma-separated registry configs (e.g. "
+                    "mononex-1b,korupel-1b,qwen3.5-0.8b): prompt and decode throughput of each instead of the headline workload")
+    ap.add_argument("--mononex-prompts", default="512,2048", help="prompt lengths of --mononex")
     args = ap.parse_args()
     if args.korupel:
         sys.exit(korupel_leg(args))
+    if args.mononex:
+        sys.exit(korupel_leg(args, args.mononex, args.mononex_prompts, "mononex"))
 
     if args.tp_inprocess:      # ranks that share a device need one hardware queue per rank stream: before the HIP runtime starts
         os.environ.setdefault("GPU_MAX_HW_QUEUES", "16")

@@ -175,6 +175,57 @@ CONFIGS.update({
 })
 
 
+# ---- layer-list decoders: Mononex ------------------------------------------------------------------------------------------
+def mononex_config(vocab: int, width: int, pattern: str, ff: int, heads: int, kv_heads: int, dim: int, vdim: int, block: int,
+                   lat_heads: int, lat_dim: int, rot_dim: int, lat_vdim: int, kv_rank: int, q_rank: int,
+                   lin_heads: int, lin_dim: int, lin_vdim: int, tau: float = 16.0, rot_base: float = 500000.0,
+                   yarn: "dict | None" = None, eps: float = 1e-5) -> dict:
+    """pattern: one letter per layer -- 'a' softmax attention inside blocks of `block` positions, 'b' the same with the keys and
+    values of the nearest 'a' before it, 'm' latent attention, 'g' gated linear attention; upper case: no feed-forward."""
+    layers, last_a = [], None
+    for i, ch in enumerate(pattern):
+        c = ch.lower()
+        if c in "ab":
+            mixer = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=dim ** -0.5, mask=dict(size=block))
+            if c == "b":
+                if last_a is None:
+                    raise ValueError("'b' needs an 'a' layer before it")
+                mixer["kv_from"] = last_a
+            else:
+                last_a = i
+            kind = "attention"
+        elif c == "m":
+            rot = dict(base=rot_base, dims=rot_dim)
+            if yarn:
+                rot["scaling"] = dict(yarn)
+            mixer = dict(heads=lat_heads, dim=lat_dim, rot_dim=rot_dim, vdim=lat_vdim, kv_rank=kv_rank, q_rank=q_rank,
+                         scale=(lat_dim + rot_dim) ** -0.5, rot=rot)
+            kind = "latent_attention"
+        elif c == "g":
+            mixer = dict(heads=lin_heads, dim=lin_dim, vdim=lin_vdim, tau=tau)
+            kind = "gla"
+        else:
+            raise ValueError(f"pattern letter {ch!r}")
+        layers.append(dict(type=kind, mixer=mixer, mlp=None if ch.isupper() else dict(kind="dense", ff=ff)))
+    return dict(architecture="Mononex", vocab=vocab, width=width, norm=dict(eps=eps), layers=layers)
+
+
+_YARN = dict(factor=4.0, original=4096, fast=32.0, slow=1.0)
+CONFIGS.update({
+    "tiny-mononex": mononex_config(320, 128, "gabMg", ff=192, heads=4, kv_heads=2, dim=32, vdim=16, block=24, lat_heads=2, lat_dim=16,
+                                   rot_dim=8, lat_vdim=24, kv_rank=32, q_rank=48, lin_heads=2, lin_dim=16, lin_vdim=32, tau=8.0,
+                                   yarn=dict(factor=2.0, original=64, fast=8.0, slow=1.0)),
+    # the widths of the Qwen3.5-0.8B text decoder (1024 wide, 3584 ff, 24 layers, vocabulary 248 320): 12 gated linear layers, 4 block
+    # attention layers with keys of their own and 4 that borrow them, 4 latent attention layers
+    "mononex-1b": mononex_config(248320, 1024, "ggabgm" * 4, ff=3584, heads=8, kv_heads=2, dim=128, vdim=128, block=4096, lat_heads=8,
+                                 lat_dim=128, rot_dim=64, lat_vdim=128, kv_rank=512, q_rank=768, lin_heads=16, lin_dim=128, lin_vdim=128,
+                                 yarn=_YARN),
+    "mononex-1b-6l": mononex_config(32768, 1024, "ggabgm", ff=3584, heads=8, kv_heads=2, dim=128, vdim=128, block=4096, lat_heads=8,
+                                    lat_dim=128, rot_dim=64, lat_vdim=128, kv_rank=512, q_rank=768, lin_heads=16, lin_dim=128, lin_vdim=128,
+                                    yarn=_YARN),
+})
+
+
 def get_config(name: str) -> dict:
     if name not in CONFIGS:
         raise KeyError(f"unknown config {name!r}; have {sorted(CONFIGS)}")

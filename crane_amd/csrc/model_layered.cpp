@@ -1069,14 +1069,22 @@ uint64_t Model::layered_decode_bytes(size_t ctx) const {
     for (size_t i = 0; i < L.spec.size(); ++i) {
         const LayerSpec& sp = L.spec[i];
         b += 2ull * (uint64_t)L.w[i].in_rows * W;
-        if (sp.mixer == LMIX_ATTN) {
-            b += 2ull * W * sp.heads * sp.dim;
-            const uint64_t seen = std::min<uint64_t>(ctx, (uint64_t)std::min<long long>(sp.win, 1ll << 40) + (uint64_t)sp.keep);
-            b += seen * (uint64_t)sp.kv_heads * sp.dim * kv_esize;
+        if (sp.mixer == LMIX_ATTN || sp.mixer == LMIX_LATENT) {
+            const uint64_t H = (uint64_t)sp.heads;
+            uint64_t row = (uint64_t)sp.kv_heads * sp.dim + (sp.own_v ? (uint64_t)sp.kv_heads * sp.vdim : 0);      // cached elements per token
+            if (sp.mixer == LMIX_LATENT) {
+                row = (uint64_t)sp.kv_rank + sp.rot_dim;
+                b += 2ull * (H * (sp.dim + sp.rot_dim) * sp.q_rank + H * sp.dim * sp.kv_rank + H * sp.vdim * sp.kv_rank);
+            }
+            b += 2ull * W * H * sp.vdim;
+            uint64_t seen = std::min<uint64_t>(ctx, (uint64_t)std::min<long long>(sp.win, 1ll << 40) + (uint64_t)sp.keep);
+            if (sp.chunk > 0) seen = std::min<uint64_t>(seen, (uint64_t)sp.chunk);
+            b += seen * row * kv_esize;
         } else {
             b += 2ull * W * sp.heads * sp.vdim + 8ull * sp.heads * sp.dim * sp.vdim;    // state read + write
+            if (sp.mixer == LMIX_GLA) b += 2ull * sp.heads * sp.dim * sp.a_rank;
         }
-        if (sp.mlp == LMLP_DENSE) b += 6ull * W * sp.ff;
+        if (sp.mlp == LMLP_DENSE) b += (sp.gated_ff ? 6ull : 4ull) * W * sp.ff;
         else if (sp.mlp == LMLP_MOE) b += 6ull * W * sp.ff * sp.top + 2ull * W * sp.experts;
     }
     return b;
