@@ -935,7 +935,8 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
         if (i < e) a.out[(size_t)row * a.ldo + head * e + i] = acc[c] * inv * (a.gate == LGATE_ELEM ? gp[i] : 1.f);
     }
 }
-// Matrix-core form for prompt passes in the bfloat16 format (head size a multiple of 16, up to 128): LAY_ATTN_MFMA_ROWS query rows per
+// Matrix-core form for prompt passes in the bfloat16 format (key and value sizes multiples of 16, up to 128; values from pages of
+// their own or the first e elements of the keys; the same masks, distance terms, sink and gates as lay_attn_kernel): LAY_ATTN_MFMA_ROWS query rows per
 // block, one wave per 16 of them, 64-key tiles (32-row blocks, two or three resident per CU, measured slower: 474 against 423 us for 2048 tokens).  S = Q K^T from the bf16-rounded q and the cached bf16 keys (exact products, f32 sums);
 // mask, distance penalty, running max / sum and the weights stay f32 as in lay_attn_kernel; the weights enter P V (V = K) as a
 // bf16 hi + lo pair, two products per tile, so that they keep 16 significand bits; exp and log are the hardware's (v_exp_f32 /
@@ -944,10 +945,11 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
 constexpr int LM_BQ = LAY_ATTN_MFMA_ROWS, LM_KT = 64, LM_NT = LM_BQ * 4, LM_NW = LM_BQ / 16;    // threads, waves
 __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-    const int d = a.d, ldq = d + 8, ldp = LM_KT + 8;
+    const int d = a.d, e = a.e, ldq = d + 8, ldp = LM_KT + 8;
+    const bool ownv = a.vpool != nullptr;
     uint16_t* Qs = smem;                              // [rows][d + 8] until the q fragments sit in registers, then:
-    uint16_t* Kt = smem;                              // [d][72] the key tile transposed (the B operand of P V: 4 keys of one element)
-    uint16_t* Ks = smem + max(LM_BQ * ldq, d * ldp);  // [64][d + 8]
+    uint16_t* Kt = smem;                              // [e][72] the value tile transposed (the B operand of P V: 4 keys of one element)
+    uint16_t* Ks = smem + max(LM_BQ * ldq, e * ldp);  // [64][d + 8]
     uint16_t* Ph = Ks + LM_KT * ldq;                  // [waves][16][72] hi
     uint16_t* Pl = Ph + LM_NW * 16 * ldp;                 // ... lo
     const int2 tile = a.tiles[blockIdx.x];
@@ -955,7 +957,7 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
     const int g = blockIdx.y, nrep = a.H / a.G;
     const int q0 = tile.y, nq = min(LM_BQ, sg.n * nrep - q0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 15, lg = lane >> 4;
-    const int win = (int)min(a.win, 1ll << 30), keep = (int)min(a.keep, 1ll << 30);
+    const int win = (int)min(a.win, 1ll << 30), keep = (int)min(a.keep, 1ll << 30), chunk = (int)min(a.chunk, 1ll << 30);
     // q rows -> bf16
     for (int idx = tid; idx < LM_BQ * (d / 4); idx += LM_NT) {
         const int qr = idx / (d / 4), i = (idx - qr * (d / 4)) * 4;
@@ -968,7 +970,8 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
         *(u32x2*)&Qs[qr * ldq + i] = pk;
     }
     // this lane's four query rows (accumulator rows 4 lg + r of the wave's 16)
-    int qpos[4], qhead[4], qrow[4]; bool qok[4]; float r1[4], r2[4];
+    int qpos[4], qhead[4], qrow[4], qclo[4]; bool qok[4]; float r1[4], r2[4];
+    float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int qr = wave * 16 + 4 * lg + r;
@@ -976,18 +979,20 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
         const int qi = q0 + (qok[r] ? qr : 0), lp = qi / nrep;
         qhead[r] = g * nrep + (qi - lp * nrep);
         qpos[r] = sg.start_pos + lp;
+        qclo[r] = chunk > 0 ? qpos[r] / chunk * chunk : 0;
         qrow[r] = sg.row0 + lp;
-        r1[r] = a.r1[qhead[r]]; r2[r] = a.r2[qhead[r]];
+        r1[r] = a.bias != LBIAS_NONE ? a.r1[qhead[r]] : 0.f; r2[r] = a.bias == LBIAS_LOG ? a.r2[qhead[r]] : 0.f;
+        if (a.sink && qok[r]) { m[r] = a.sink[qhead[r]]; l[r] = 1.f; }      // exp(sink - m) with m = sink
     }
     const int pmin = sg.start_pos + q0 / nrep, pmax = sg.start_pos + (q0 + nq - 1) / nrep;
-    const int main_lo = max(0, pmin - win + 1);
+    int main_lo = max(0, pmin - win + 1);
+    if (chunk > 0) main_lo = max(main_lo, pmin / chunk * chunk);
     const int sink_hi = min(keep, main_lo);
     const int total = sink_hi + (pmax - main_lo + 1);
     f32x4 O[8];
 #pragma unroll
     for (int n = 0; n < 8; ++n) O[n] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
-    const int nd = d / 16;
+    const int nd = d / 16, ne = e / 16;
     uint16_t* ph = Ph + wave * 16 * ldp;
     uint16_t* pl = Pl + wave * 16 * ldp;
     __syncthreads();                       // Qs written
@@ -1007,11 +1012,28 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
                 pk = *(const u32x4*)((const uint16_t*)a.kpool + (((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * d + i);
             }
             *(u32x4*)&Ks[sl * ldq + i] = pk;
-            Kt[(i + 0) * ldp + sl] = (uint16_t)(pk.x & 0xFFFFu); Kt[(i + 1) * ldp + sl] = (uint16_t)(pk.x >> 16);
-            Kt[(i + 2) * ldp + sl] = (uint16_t)(pk.y & 0xFFFFu); Kt[(i + 3) * ldp + sl] = (uint16_t)(pk.y >> 16);
-            Kt[(i + 4) * ldp + sl] = (uint16_t)(pk.z & 0xFFFFu); Kt[(i + 5) * ldp + sl] = (uint16_t)(pk.z >> 16);
-            Kt[(i + 6) * ldp + sl] = (uint16_t)(pk.w & 0xFFFFu); Kt[(i + 7) * ldp + sl] = (uint16_t)(pk.w >> 16);
+            if (!ownv && i < e) {
+                Kt[(i + 0) * ldp + sl] = (uint16_t)(pk.x & 0xFFFFu); Kt[(i + 1) * ldp + sl] = (uint16_t)(pk.x >> 16);
+                Kt[(i + 2) * ldp + sl] = (uint16_t)(pk.y & 0xFFFFu); Kt[(i + 3) * ldp + sl] = (uint16_t)(pk.y >> 16);
+                Kt[(i + 4) * ldp + sl] = (uint16_t)(pk.z & 0xFFFFu); Kt[(i + 5) * ldp + sl] = (uint16_t)(pk.z >> 16);
+                Kt[(i + 6) * ldp + sl] = (uint16_t)(pk.w & 0xFFFFu); Kt[(i + 7) * ldp + sl] = (uint16_t)(pk.w >> 16);
+            }
         }
+        if (ownv)
+            for (int idx = tid; idx < LM_KT * (e / 8); idx += LM_NT) {
+                const int sl = idx / (e / 8), i = (idx - sl * (e / 8)) * 8;
+                const int v = v0 + sl;
+                u32x4 pk = {0u, 0u, 0u, 0u};
+                if (v < total) {
+                    const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
+                    const int pg = a.bt[sg.bt_off + j / a.page];
+                    pk = *(const u32x4*)((const uint16_t*)a.vpool + (((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * e + i);
+                }
+                Kt[(i + 0) * ldp + sl] = (uint16_t)(pk.x & 0xFFFFu); Kt[(i + 1) * ldp + sl] = (uint16_t)(pk.x >> 16);
+                Kt[(i + 2) * ldp + sl] = (uint16_t)(pk.y & 0xFFFFu); Kt[(i + 3) * ldp + sl] = (uint16_t)(pk.y >> 16);
+                Kt[(i + 4) * ldp + sl] = (uint16_t)(pk.z & 0xFFFFu); Kt[(i + 5) * ldp + sl] = (uint16_t)(pk.z >> 16);
+                Kt[(i + 6) * ldp + sl] = (uint16_t)(pk.w & 0xFFFFu); Kt[(i + 7) * ldp + sl] = (uint16_t)(pk.w >> 16);
+            }
         __syncthreads();
         f32x4 S[4];
 #pragma unroll
@@ -1035,8 +1057,9 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
                 const int v = v0 + t * 16 + lr;
                 const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
                 const int dist = qpos[r] - j;
-                const bool vis = qok[r] && v < total && dist >= 0 && (dist < win || j < keep);
-                sc[t] = vis ? S[t][r] * a.scale - r1[r] * __logf(1.f + r2[r] * (float)dist) : -INFINITY;
+                const bool vis = qok[r] && v < total && dist >= 0 && ((dist < win && j >= qclo[r]) || j < keep);
+                const float pen = a.bias == LBIAS_LOG ? r1[r] * __logf(1.f + r2[r] * (float)dist) : r1[r] * (float)dist;
+                sc[t] = vis ? S[t][r] * a.scale - pen : -INFINITY;
                 tmax = fmaxf(tmax, sc[t]);
             }
             tmax = row16_max(tmax);
@@ -1066,7 +1089,7 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
             const bf16x4 al = *(const bf16x4*)&pl[lr * ldp + ks * 16 + 4 * lg];
 #pragma unroll
             for (int n = 0; n < 8; ++n) {
-                if (n < nd) {
+                if (n < ne) {
                     const bf16x4 vb = *(const bf16x4*)&Kt[(n * 16 + lr) * ldp + ks * 16 + 4 * lg];
                     O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah, vb, O[n], 0, 0, 0);
                     O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(al, vb, O[n], 0, 0, 0);
@@ -1077,15 +1100,19 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         if (!qok[r]) continue;
-        const float inv = a.proj[(size_t)qrow[r] * a.ldp + a.g_off + qhead[r]] / l[r];
+        const float* gp = a.proj + (size_t)qrow[r] * a.ldp + a.g_off + (a.gate == LGATE_ELEM ? qhead[r] * e : qhead[r]);
+        const float inv = (a.gate == LGATE_HEAD ? gp[0] : 1.f) / l[r];
 #pragma unroll
         for (int n = 0; n < 8; ++n)
-            if (n < nd) a.out[(size_t)qrow[r] * a.ldo + qhead[r] * d + n * 16 + lr] = O[n][r] * inv;
+            if (n < ne) a.out[(size_t)qrow[r] * a.ldo + qhead[r] * e + n * 16 + lr] = O[n][r] * inv * (a.gate == LGATE_ELEM ? gp[n * 16 + lr] : 1.f);
     }
 }
-void launch_lay_attn_mfma(const LAttnArgs& a, hipStream_t s) {
-    if (a.ntiles <= 0) return;
-    const size_t lds = ((size_t)std::max(LM_BQ * (a.d + 8), a.d * (LM_KT + 8)) + (size_t)LM_KT * (a.d + 8) + 2 * LM_NW * 16 * (LM_KT + 8)) * sizeof(uint16_t);
+bool lay_attn_mfma_fits(int d, int e) { return d % 16 == 0 && e % 16 == 0 && d <= 128 && e <= 128 && d > 0 && e > 0; }
+void launch_lay_attn_mfma(const LAttnArgs& a0, hipStream_t s) {
+    if (a0.ntiles <= 0) return;
+    LAttnArgs a = a0;
+    if (a.e <= 0) a.e = a.d;
+    const size_t lds = ((size_t)std::max(LM_BQ * (a.d + 8), a.e * (LM_KT + 8)) + (size_t)LM_KT * (a.d + 8) + 2 * LM_NW * 16 * (LM_KT + 8)) * sizeof(uint16_t);
     hipLaunchKernelGGL(lay_attn_mfma_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(LM_NT), lds, s, a);
 }
 

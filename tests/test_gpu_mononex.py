@@ -498,3 +498,33 @@ def test_a_step_larger_than_one_pass_is_cut_into_passes(tmp_path):
         assert [m.seq_len(x) for x in s] == [100, 45, 9]
     finally:
         m.close()
+
+
+def test_matrix_core_attention_of_prompt_passes(tmp_path):
+    """bfloat16 format, key and value sizes that are multiples of 16: prompt passes run block attention (value pages of their own,
+    block edges inside a tile, the sink, borrowed pages) and latent attention (values = the latent part of the cached rows) on the
+    matrix cores.  Against the oracle, and against the same steps with the switch off."""
+    cfg = U.config([U.layer("attention", U.dense(), **U.attn(heads=6, kv_heads=2, dim=32, vdim=16, size=50)),
+                    U.layer("latent_attention", None, **U.latent(heads=3, dim=16, rot_dim=16, vdim=24, kv_rank=48, q_rank=40)),
+                    U.layer("attention", None, **U.attn(heads=2, kv_heads=2, dim=32, vdim=16, size=7, scale=0.4, kv_from=0)),
+                    U.layer("attention", None, **U.attn(heads=5, kv_heads=1, dim=16, vdim=48, size=None))], vocab=90, width=64)
+    P = U.random_weights(cfg, 18)
+    reqs = [U.tokens(200, cfg["vocab"], 81), U.tokens(90, cfg["vocab"], 82)]
+    want = [O.forward(cfg, P, t) for t in reqs]
+    m = _load(tmp_path, cfg, P, dtype="bfloat16")
+    try:
+        outs = []
+        for on in (1, 0):
+            m.debug_set("lay_attn_mfma", on)
+            a, b = m.seq_alloc(), m.seq_alloc()
+            g1, _ = m.step_batch([(a, reqs[0][:130], _all(130)), (b, reqs[1][:17], _all(17))])
+            g2, _ = m.step_batch([(a, reqs[0][130:], _all(70)), (b, reqs[1][17:], _all(73))])
+            got = [np.concatenate([g1[:130], g2[:70]]), np.concatenate([g1[130:], g2[70:]])]
+            for r in range(2):
+                assert _err(got[r], want[r]) < TOL_BF16, (on, r)
+            outs.append(got)
+            m.seq_free(a); m.seq_free(b)
+        for r in range(2):
+            assert _err(outs[0][r], outs[1][r]) < 3e-2
+    finally:
+        m.close()
