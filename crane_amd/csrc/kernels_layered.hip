@@ -809,6 +809,7 @@ void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int
 // ([..][e]) or the first e elements of the key rows.  A sink adds exp(sink) to the denominator: it is the start value of the running
 // (max, sum) pair of the first split.  Scores, softmax and the weighted sum are f32.
 constexpr int LA_BQ = 16;
+constexpr size_t LDS_PLAIN = 64 * 1024, LDS_MAX = 160 * 1024;    // without / with the kernel's dynamic-LDS attribute raised
 template <int KVT, int KT, int NACC>
 __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
     extern __shared__ float lds[];
@@ -943,13 +944,17 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
 // v_log_f32, about 1e-6 relative: the format's own rounding is three orders above that).  Fragment layout of v_mfma_f32_16x16x16_bf16:
 // A[i = lane % 16][k = 4 (lane / 16) ..], B[k = 4 (lane / 16) ..][j = lane % 16], D[i = 4 (lane / 16) + r][j = lane % 16].
 constexpr int LM_BQ = LAY_ATTN_MFMA_ROWS, LM_KT = 64, LM_NT = LM_BQ * 4, LM_NW = LM_BQ / 16;    // threads, waves
+// NDMAX / NEMAX: key / value size in units of 16 the registers are laid out for (q fragments, output tiles).  WIDE: long cached rows
+// whose values are their own first e elements (latent attention: [latent | rotated key part]); the key tile takes the place of the
+// staged queries, and the B operand of P V (4 keys of one element) is gathered from the key rows instead of a transposed copy.
+template <int NDMAX, int NEMAX, bool WIDE>
 __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
     const int d = a.d, e = a.e, ldq = d + 8, ldp = LM_KT + 8;
     const bool ownv = a.vpool != nullptr;
     uint16_t* Qs = smem;                              // [rows][d + 8] until the q fragments sit in registers, then:
     uint16_t* Kt = smem;                              // [e][72] the value tile transposed (the B operand of P V: 4 keys of one element)
-    uint16_t* Ks = smem + max(LM_BQ * ldq, e * ldp);  // [64][d + 8]
+    uint16_t* Ks = WIDE ? smem : smem + max(LM_BQ * ldq, e * ldp);  // [64][d + 8]
     uint16_t* Ph = Ks + LM_KT * ldq;                  // [waves][16][72] hi
     uint16_t* Pl = Ph + LM_NW * 16 * ldp;                 // ... lo
     const int2 tile = a.tiles[blockIdx.x];
@@ -989,16 +994,16 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
     if (chunk > 0) main_lo = max(main_lo, pmin / chunk * chunk);
     const int sink_hi = min(keep, main_lo);
     const int total = sink_hi + (pmax - main_lo + 1);
-    f32x4 O[8];
+    f32x4 O[NEMAX];
 #pragma unroll
-    for (int n = 0; n < 8; ++n) O[n] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int n = 0; n < NEMAX; ++n) O[n] = (f32x4){0.f, 0.f, 0.f, 0.f};
     const int nd = d / 16, ne = e / 16;
     uint16_t* ph = Ph + wave * 16 * ldp;
     uint16_t* pl = Pl + wave * 16 * ldp;
     __syncthreads();                       // Qs written
-    bf16x4 qf[8];
+    bf16x4 qf[NDMAX];
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk)
+    for (int kk = 0; kk < NDMAX; ++kk)
         qf[kk] = kk < nd ? *(const bf16x4*)&Qs[(wave * 16 + lr) * ldq + kk * 16 + 4 * lg] : (bf16x4){0, 0, 0, 0};
     for (int v0 = 0; v0 < total; v0 += LM_KT) {
         __syncthreads();                   // previous tile consumed (first round: q fragments read, Qs free for Kt)
@@ -1012,14 +1017,14 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
                 pk = *(const u32x4*)((const uint16_t*)a.kpool + (((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * d + i);
             }
             *(u32x4*)&Ks[sl * ldq + i] = pk;
-            if (!ownv && i < e) {
+            if (!WIDE && !ownv && i < e) {
                 Kt[(i + 0) * ldp + sl] = (uint16_t)(pk.x & 0xFFFFu); Kt[(i + 1) * ldp + sl] = (uint16_t)(pk.x >> 16);
                 Kt[(i + 2) * ldp + sl] = (uint16_t)(pk.y & 0xFFFFu); Kt[(i + 3) * ldp + sl] = (uint16_t)(pk.y >> 16);
                 Kt[(i + 4) * ldp + sl] = (uint16_t)(pk.z & 0xFFFFu); Kt[(i + 5) * ldp + sl] = (uint16_t)(pk.z >> 16);
                 Kt[(i + 6) * ldp + sl] = (uint16_t)(pk.w & 0xFFFFu); Kt[(i + 7) * ldp + sl] = (uint16_t)(pk.w >> 16);
             }
         }
-        if (ownv)
+        if (!WIDE && ownv)
             for (int idx = tid; idx < LM_KT * (e / 8); idx += LM_NT) {
                 const int sl = idx / (e / 8), i = (idx - sl * (e / 8)) * 8;
                 const int v = v0 + sl;
@@ -1039,13 +1044,14 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-            if (kk >= nd) break;
-            const bf16x4 qa = qf[kk];
+        for (int kk = 0; kk < NDMAX; ++kk) {
+            if (kk < nd) {
+                const bf16x4 qa = qf[kk];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const bf16x4 kb = *(const bf16x4*)&Ks[(t * 16 + lr) * ldq + kk * 16 + 4 * lg];
-                S[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(qa, kb, S[t], 0, 0, 0);
+                for (int t = 0; t < 4; ++t) {
+                    const bf16x4 kb = *(const bf16x4*)&Ks[(t * 16 + lr) * ldq + kk * 16 + 4 * lg];
+                    S[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(qa, kb, S[t], 0, 0, 0);
+                }
             }
         }
         float corr[4];
@@ -1079,7 +1085,7 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
             m[r] = mn;
         }
 #pragma unroll
-        for (int n = 0; n < 8; ++n)
+        for (int n = 0; n < NEMAX; ++n)
 #pragma unroll
             for (int r = 0; r < 4; ++r) O[n][r] *= corr[r];
         __syncthreads();                   // the wave's weights are in LDS
@@ -1088,9 +1094,13 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
             const bf16x4 ah = *(const bf16x4*)&ph[lr * ldp + ks * 16 + 4 * lg];
             const bf16x4 al = *(const bf16x4*)&pl[lr * ldp + ks * 16 + 4 * lg];
 #pragma unroll
-            for (int n = 0; n < 8; ++n) {
+            for (int n = 0; n < NEMAX; ++n) {
                 if (n < ne) {
-                    const bf16x4 vb = *(const bf16x4*)&Kt[(n * 16 + lr) * ldp + ks * 16 + 4 * lg];
+                    bf16x4 vb;
+                    if (WIDE) {
+                        const uint16_t* kc = Ks + (ks * 16 + 4 * lg) * ldq + n * 16 + lr;
+                        vb = (bf16x4){(short)kc[0], (short)kc[ldq], (short)kc[2 * ldq], (short)kc[3 * ldq]};
+                    } else vb = *(const bf16x4*)&Kt[(n * 16 + lr) * ldp + ks * 16 + 4 * lg];
                     O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah, vb, O[n], 0, 0, 0);
                     O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(al, vb, O[n], 0, 0, 0);
                 }
@@ -1103,17 +1113,40 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
         const float* gp = a.proj + (size_t)qrow[r] * a.ldp + a.g_off + (a.gate == LGATE_ELEM ? qhead[r] * e : qhead[r]);
         const float inv = (a.gate == LGATE_HEAD ? gp[0] : 1.f) / l[r];
 #pragma unroll
-        for (int n = 0; n < 8; ++n)
+        for (int n = 0; n < NEMAX; ++n)
             if (n < ne) a.out[(size_t)qrow[r] * a.ldo + qhead[r] * e + n * 16 + lr] = O[n][r] * inv * (a.gate == LGATE_ELEM ? gp[n * 16 + lr] : 1.f);
     }
 }
-bool lay_attn_mfma_fits(int d, int e) { return d % 16 == 0 && e % 16 == 0 && d <= 128 && e <= 128 && d > 0 && e > 0; }
+bool lay_attn_mfma_fits(int d, int e, bool own_v) {
+    if (d <= 0 || e <= 0 || d % 16 || e % 16) return false;
+    if (d <= 128 && e <= 128) return own_v || e <= d;
+    return !own_v && e <= d && d <= 640 && e <= 512;      // the wide form
+}
+template <int NDMAX, int NEMAX, bool WIDE>
+static void lay_attn_mfma_go(const LAttnArgs& a, size_t lds, hipStream_t s) {
+    if (lds > LDS_PLAIN) {
+        static bool raised = false;        // per instantiation
+        if (!raised) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&lay_attn_mfma_kernel<NDMAX, NEMAX, WIDE>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL((lay_attn_mfma_kernel<NDMAX, NEMAX, WIDE>), dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(LM_NT), lds, s, a);
+}
 void launch_lay_attn_mfma(const LAttnArgs& a0, hipStream_t s) {
     if (a0.ntiles <= 0) return;
     LAttnArgs a = a0;
     if (a.e <= 0) a.e = a.d;
-    const size_t lds = ((size_t)std::max(LM_BQ * (a.d + 8), a.e * (LM_KT + 8)) + (size_t)LM_KT * (a.d + 8) + 2 * LM_NW * 16 * (LM_KT + 8)) * sizeof(uint16_t);
-    hipLaunchKernelGGL(lay_attn_mfma_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(LM_NT), lds, s, a);
+    const size_t pbytes = (size_t)2 * LM_NW * 16 * (LM_KT + 8);
+    if (a.d <= 128 && a.e <= 128) {
+        const size_t lds = ((size_t)std::max(LM_BQ * (a.d + 8), a.e * (LM_KT + 8)) + (size_t)LM_KT * (a.d + 8) + pbytes) * sizeof(uint16_t);
+        lay_attn_mfma_go<8, 8, false>(a, lds, s);
+        return;
+    }
+    const size_t lds = ((size_t)std::max(LM_BQ, LM_KT) * (a.d + 8) + pbytes) * sizeof(uint16_t);
+    if (a.d <= 320 && a.e <= 256) lay_attn_mfma_go<20, 16, true>(a, lds, s);
+    else lay_attn_mfma_go<40, 32, true>(a, lds, s);
 }
 
 // merge of the splits of a tile: out = sum_z acc_z e^(m_z - M) / sum_z l_z e^(m_z - M) * gate; one thread per (query row, element)
@@ -1145,7 +1178,6 @@ __global__ __launch_bounds__(256) void lay_attn_merge_kernel(LAttnArgs a, int ns
 static size_t lay_attn_lds(int d, int e, bool own_v, int KT) {
     return (size_t)(LA_BQ * d + KT * (d + 1) + (own_v ? KT * e : 0) + LA_BQ * KT) * sizeof(float);
 }
-constexpr size_t LDS_PLAIN = 64 * 1024, LDS_MAX = 160 * 1024;    // without / with the kernel's dynamic-LDS attribute raised
 bool lay_attn_fits(int d, int e, bool own_v) {
     return d > 0 && e > 0 && e <= 512 && (own_v || e <= d) && lay_attn_lds(d, e, own_v, 32) <= LDS_MAX;
 }

@@ -171,7 +171,7 @@ bool lay_attn_fits(int d, int e, bool own_v);                         // sizes t
 // LAY_ATTN_MFMA_ROWS rows, longest key range first
 constexpr int LAY_ATTN_MFMA_ROWS = 64;
 void launch_lay_attn_mfma(const LAttnArgs& a, hipStream_t s);
-bool lay_attn_mfma_fits(int d, int e);
+bool lay_attn_mfma_fits(int d, int e, bool own_v);         // sizes the matrix-core form takes
 
 struct LLightArgs {
     const float* proj; int ldp, q_off, k_off, v_off; // activated projection rows

@@ -863,7 +863,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 a.nsplit = std::max(1, std::min({32, key_tiles, 256 / blocks, Layered::ATT_PARTS / blocks}));
                 a.part_o = L.att_po; a.part_ml = L.att_pml;
             }
-            if (L.attn_mfma && kv_mode == KV_BF16 && !all_decode && max_n >= 16 && lay_attn_mfma_fits(dk, ev) && (a.vpool || ev <= dk)) {
+            if (L.attn_mfma && kv_mode == KV_BF16 && !all_decode && max_n >= 16 && lay_attn_mfma_fits(dk, ev, a.vpool != nullptr)) {
                 const auto& tm = tiles64[sp.heads / sp.kv_heads];
                 a.tiles = (const int2*)(L.d_tab + tm.first); a.ntiles = tm.second;
                 launch_lay_attn_mfma(a, s);

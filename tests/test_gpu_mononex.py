@@ -528,3 +528,31 @@ def test_matrix_core_attention_of_prompt_passes(tmp_path):
             assert _err(outs[0][r], outs[1][r]) < 3e-2
     finally:
         m.close()
+
+
+def test_matrix_core_latent_attention_over_long_cached_rows(tmp_path):
+    """bfloat16 format, cached rows of 192 and 288 elements (latent + rotated key part): the wide matrix-core form of prompt
+    passes (the value operand gathered from the key rows), both register layouts.  Against the oracle and against the switch off."""
+    cfg = U.config([U.layer("latent_attention", U.dense(), **U.latent(heads=3, dim=16, rot_dim=16, vdim=24, kv_rank=176, q_rank=40, scale=0.1)),
+                    U.layer("latent_attention", None, **U.latent(heads=2, dim=8, rot_dim=16, vdim=16, kv_rank=272, q_rank=24, scale=0.1))],
+                   vocab=90, width=64)
+    P = U.random_weights(cfg, 19)
+    reqs = [U.tokens(150, cfg["vocab"], 83), U.tokens(70, cfg["vocab"], 84)]
+    want = [O.forward(cfg, P, t) for t in reqs]
+    m = _load(tmp_path, cfg, P, dtype="bfloat16")
+    try:
+        outs = []
+        for on in (1, 0):
+            m.debug_set("lay_attn_mfma", on)
+            a, b = m.seq_alloc(), m.seq_alloc()
+            g1, _ = m.step_batch([(a, reqs[0][:100], _all(100)), (b, reqs[1][:17], _all(17))])
+            g2, _ = m.step_batch([(a, reqs[0][100:], _all(50)), (b, reqs[1][17:], _all(53))])
+            got = [np.concatenate([g1[:100], g2[:50]]), np.concatenate([g1[100:], g2[50:]])]
+            for r in range(2):
+                assert _err(got[r], want[r]) < TOL_BF16, (on, r)
+            outs.append(got)
+            m.seq_free(a); m.seq_free(b)
+        for r in range(2):
+            assert _err(outs[0][r], outs[1][r]) < 3e-2
+    finally:
+        m.close()
