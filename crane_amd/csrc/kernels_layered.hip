@@ -1405,27 +1405,19 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
     float* bs = pw + LC + 1;               // gated: [LC][d + 1]
     const int2 ch = a.chunks[blockIdx.x];
     const LaySegDev sg = a.segs[ch.x];
-    const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
-    const int ne = min(LL_ES, e - j0), n = min(LC, sg.n - ch.y);
+    const int head = blockIdx.y, tid = threadIdx.x;
+    const int n = min(LC, sg.n - ch.y);
     if (!GT) {
         const float decay = a.decay[head];
         if (tid <= LC) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
     }
     const float* U = a.U + ((size_t)blockIdx.x * a.H + head) * d * e;
-    for (int idx = tid; idx < d * LL_ES; idx += 256) {
-        const int i = idx / LL_ES, j = idx % LL_ES;
-        S[idx] = j < ne ? U[(size_t)i * e + j0 + j] : 0.f;
-    }
     for (int idx = tid; idx < n * d; idx += 256) {
         const int t = idx / d, i = idx - t * d;
         const size_t base = (size_t)(sg.row0 + ch.y + t) * a.ldp + (size_t)head * d + i;
         qs[idx] = a.proj[base + a.q_off] * a.qscale;
         ks[t * ldk + i] = a.proj[base + a.k_off];
         if (GT) bs[t * ldk + i] = a.ldec[(size_t)(sg.row0 + ch.y + t) * a.ldd + (size_t)head * d + i];
-    }
-    for (int idx = tid; idx < n * LL_ES; idx += 256) {
-        const int t = idx / LL_ES, j = idx % LL_ES;
-        vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
     }
     __syncthreads();
     if (GT) {
@@ -1451,15 +1443,29 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
     __syncthreads();
     if (GT) {
         for (int idx = tid; idx < n * d; idx += 256) { const int t = idx / d, i = idx - t * d; qs[idx] *= expf(bs[t * ldk + i]); }
-        __syncthreads();
     }
-    for (int idx = tid; idx < n * LL_ES; idx += 256) {
-        const int t = idx / LL_ES, j = idx % LL_ES;
-        float inter = 0.f;
-        for (int i = 0; i < d; ++i) inter = fmaf(S[i * LL_ES + j], qs[t * d + i], inter);
-        float o = GT ? inter : inter * pw[t + 1];
-        for (int s = 0; s <= t; ++s) o = fmaf(As[t * LC + s], vs[s * LL_ES + j], o);
-        if (j < ne) a.out[(size_t)(sg.row0 + ch.y + t) * a.ldo + (size_t)head * e + j0 + j] = o;
+    // value slices: the launch's z blocks take them in turn (gated form: one block walks all of them, the scores above are its
+    // expensive part and do not depend on the slice)
+    for (int j0 = blockIdx.z * LL_ES; j0 < e; j0 += gridDim.z * LL_ES) {
+        const int ne = min(LL_ES, e - j0);
+        __syncthreads();                   // the previous slice is written out; qs / As complete
+        for (int idx = tid; idx < d * LL_ES; idx += 256) {
+            const int i = idx / LL_ES, j = idx % LL_ES;
+            S[idx] = j < ne ? U[(size_t)i * e + j0 + j] : 0.f;
+        }
+        for (int idx = tid; idx < n * LL_ES; idx += 256) {
+            const int t = idx / LL_ES, j = idx % LL_ES;
+            vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < n * LL_ES; idx += 256) {
+            const int t = idx / LL_ES, j = idx % LL_ES;
+            float inter = 0.f;
+            for (int i = 0; i < d; ++i) inter = fmaf(S[i * LL_ES + j], qs[t * d + i], inter);
+            float o = GT ? inter : inter * pw[t + 1];
+            for (int s = 0; s <= t; ++s) o = fmaf(As[t * LC + s], vs[s * LL_ES + j], o);
+            if (j < ne) a.out[(size_t)(sg.row0 + ch.y + t) * a.ldo + (size_t)head * e + j0 + j] = o;
+        }
     }
 }
 
@@ -1518,7 +1524,9 @@ static void lay_lightning_go(const LLightArgs& a, hipStream_t s) {
         ll_raise_lds(lay_light_chunk_out_kernel<GT>, l3);
         hipLaunchKernelGGL(lay_light_chunk_kv_kernel<GT>, gc, dim3(256), l1, s, a);
         hipLaunchKernelGGL(lay_light_scan_kernel<GT>, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.d * a.e + 255) / 256)), dim3(256), 0, s, a);
-        hipLaunchKernelGGL(lay_light_chunk_out_kernel<GT>, gc, dim3(256), l3, s, a);
+        // gated form: one block per (chunk, head) once the launch fills the chip without the split over value slices
+        const dim3 go(gc.x, gc.y, GT && gc.x * gc.y >= 512 ? 1u : gc.z);
+        hipLaunchKernelGGL(lay_light_chunk_out_kernel<GT>, go, dim3(256), l3, s, a);
         return;
     }
     const int C = a.d > 128 ? 8 : 16;

@@ -84,6 +84,18 @@ static void lay_gemm(Model& m, Layered& L, const LGemmArgs& g, int groups, hipSt
             return;
         }
     }
+    // a wide product whose column count is no multiple of the shared GEMM's tile: the whole tiles there, the last columns here
+    if (bf && L.shared_gemm && L.Abf && groups == 1 && !g.a_idx && !g.c_idx && !g.grp_off && !g.mul && !g.W2 && g.M >= 256 && g.N >= 256 &&
+        g.N % 128 != 0 && g.K % 32 == 0) {
+        const int n0 = g.N - g.N % 128;
+        LGemmArgs g1 = g, g2 = g;
+        g1.N = n0;
+        g2.W = g.W + (size_t)n0 * g.K; g2.C = g.C + n0; g2.N = g.N - n0; g2.bias = g.bias ? g.bias + n0 : nullptr;
+        g2.act_split = std::max(0, g.act_split - n0);
+        lay_gemm(m, L, g1, 1, s);
+        launch_lgemm(g2, bf, 1, s);
+        return;
+    }
     launch_lgemm(g, bf, groups, s);
 }
 

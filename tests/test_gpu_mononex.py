@@ -433,22 +433,22 @@ def test_synthetic_registry_model_generates(tmp_path):
 
 
 def test_bfloat16_products_on_the_shared_gemm_and_on_the_row_kernel_agree(tmp_path):
-    """Widths that fit the matrix-core GEMM of the other families (output widths that are multiples of 128): a 100-token prompt
+    """Widths that fit the matrix-core GEMM of the other families (output widths that are multiples of 128): a 300-token prompt
     (shared GEMM for the products that fit), the same with the switch off (tiled kernel of this family), and token by token
     (row kernel)."""
     cfg = U.config([U.layer("attention", U.dense(256), **U.attn(heads=4, kv_heads=2, dim=32, vdim=32, size=40)),
-                    U.layer("gla", U.dense(256), **U.gla(heads=2, dim=16, vdim=32, tau=8.0)),
+                    U.layer("gla", U.dense(256), **U.gla(heads=2, dim=32, vdim=64, tau=8.0)),      # 416 input-projection columns: 384 + 32
                     U.layer("latent_attention", U.dense(128), **U.latent(heads=4, dim=16, rot_dim=16, vdim=32, kv_rank=32, q_rank=64)),
                     U.layer("attention", None, **U.attn(heads=4, kv_heads=2, dim=32, vdim=32, size=24, kv_from=0))], vocab=320, width=128)
     P = U.random_weights(cfg, 15, a_rank=32)
-    toks = U.tokens(100, cfg["vocab"], 15)
+    toks = U.tokens(300, cfg["vocab"], 15)                         # 256 rows and more: wide products are split at the last whole tile
     want = O.forward(cfg, P, toks)
     m = _load(tmp_path, cfg, P, dtype="bfloat16")
     try:
         a, b, c = m.seq_alloc(), m.seq_alloc(), m.seq_alloc()
-        shared, _ = m.step_batch([(a, toks, _all(100))])
+        shared, _ = m.step_batch([(a, toks, _all(300))])
         m.debug_set("lay_shared_gemm", 0)
-        tiled, _ = m.step_batch([(b, toks, _all(100))])
+        tiled, _ = m.step_batch([(b, toks, _all(300))])
         rows = np.concatenate([m.step_batch([(c, [t], [0])])[0] for t in toks])
         for got in (shared, tiled, rows):
             assert _err(got, want) < TOL_BF16
@@ -554,5 +554,21 @@ def test_matrix_core_latent_attention_over_long_cached_rows(tmp_path):
             m.seq_free(a); m.seq_free(b)
         for r in range(2):
             assert _err(outs[0][r], outs[1][r]) < 3e-2
+    finally:
+        m.close()
+
+
+def test_gated_linear_attention_over_a_whole_pass_of_chunks(tmp_path):
+    """2048 + 37 tokens, 8 heads: the first pass has 512 (chunk, head) pairs, where one block walks all value slices of its pair."""
+    cfg = U.config([U.layer("gla", None, **U.gla(heads=8, dim=8, vdim=40, tau=5.0))], vocab=53, width=32)
+    P = U.random_weights(cfg, 20)
+    toks = U.tokens(2085, cfg["vocab"], 20)
+    want = O.forward(cfg, P, toks)
+    rows = [0, 31, 32, 1000, 2047, 2048, 2084]
+    m = _load(tmp_path, cfg, P, max_seq_len=2112, kv_pool_tokens=2112)
+    try:
+        s = m.seq_alloc()
+        got, _ = m.step_batch([(s, toks, rows)])
+        assert _err(got, want[rows]) < TOL_F32
     finally:
         m.close()
