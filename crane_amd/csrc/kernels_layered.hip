@@ -1412,6 +1412,21 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
         if (tid <= LC) pw[tid] = tid == 0 ? 1.f : powf(decay, (float)tid);
     }
     const float* U = a.U + ((size_t)blockIdx.x * a.H + head) * d * e;
+    // value slices: the launch's z blocks take them in turn (gated form: one block may walk all of them -- the scores are its
+    // expensive part and do not depend on the slice); the first slice's state and values are requested with q and k
+    int j0 = blockIdx.z * LL_ES;
+    auto load_slice = [&]() {
+        const int ne = min(LL_ES, e - j0);
+        for (int idx = tid; idx < d * LL_ES; idx += 256) {
+            const int i = idx / LL_ES, j = idx % LL_ES;
+            S[idx] = j < ne ? U[(size_t)i * e + j0 + j] : 0.f;
+        }
+        for (int idx = tid; idx < n * LL_ES; idx += 256) {
+            const int t = idx / LL_ES, j = idx % LL_ES;
+            vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+        }
+    };
+    load_slice();
     for (int idx = tid; idx < n * d; idx += 256) {
         const int t = idx / d, i = idx - t * d;
         const size_t base = (size_t)(sg.row0 + ch.y + t) * a.ldp + (size_t)head * d + i;
@@ -1443,21 +1458,10 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
     __syncthreads();
     if (GT) {
         for (int idx = tid; idx < n * d; idx += 256) { const int t = idx / d, i = idx - t * d; qs[idx] *= expf(bs[t * ldk + i]); }
-    }
-    // value slices: the launch's z blocks take them in turn (gated form: one block walks all of them, the scores above are its
-    // expensive part and do not depend on the slice)
-    for (int j0 = blockIdx.z * LL_ES; j0 < e; j0 += gridDim.z * LL_ES) {
-        const int ne = min(LL_ES, e - j0);
-        __syncthreads();                   // the previous slice is written out; qs / As complete
-        for (int idx = tid; idx < d * LL_ES; idx += 256) {
-            const int i = idx / LL_ES, j = idx % LL_ES;
-            S[idx] = j < ne ? U[(size_t)i * e + j0 + j] : 0.f;
-        }
-        for (int idx = tid; idx < n * LL_ES; idx += 256) {
-            const int t = idx / LL_ES, j = idx % LL_ES;
-            vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
-        }
         __syncthreads();
+    }
+    for (;;) {
+        const int ne = min(LL_ES, e - j0);
         for (int idx = tid; idx < n * LL_ES; idx += 256) {
             const int t = idx / LL_ES, j = idx % LL_ES;
             float inter = 0.f;
@@ -1466,6 +1470,12 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
             for (int s = 0; s <= t; ++s) o = fmaf(As[t * LC + s], vs[s * LL_ES + j], o);
             if (j < ne) a.out[(size_t)(sg.row0 + ch.y + t) * a.ldo + (size_t)head * e + j0 + j] = o;
         }
+        if (!GT) break;                    // every slice has its own block: straight-line code
+        j0 += gridDim.z * LL_ES;
+        if (j0 >= e) break;
+        __syncthreads();                   // this slice's state and values are no longer read
+        load_slice();
+        __syncthreads();
     }
 }
 
@@ -1525,7 +1535,7 @@ static void lay_lightning_go(const LLightArgs& a, hipStream_t s) {
         hipLaunchKernelGGL(lay_light_chunk_kv_kernel<GT>, gc, dim3(256), l1, s, a);
         hipLaunchKernelGGL(lay_light_scan_kernel<GT>, dim3((unsigned)a.nseg, (unsigned)a.H, (unsigned)((a.d * a.e + 255) / 256)), dim3(256), 0, s, a);
         // gated form: one block per (chunk, head) once the launch fills the chip without the split over value slices
-        const dim3 go(gc.x, gc.y, GT && gc.x * gc.y >= 512 ? 1u : gc.z);
+        const dim3 go(gc.x, gc.y, GT && gc.x * gc.y >= 512 ? 1u : gc.z);      // the plain form keeps one block per slice
         hipLaunchKernelGGL(lay_light_chunk_out_kernel<GT>, go, dim3(256), l3, s, a);
         return;
     }
