@@ -815,10 +815,11 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
     extern __shared__ float lds[];
     const int d = a.d, e = a.e, ldk = d + 1;
     const bool ownv = a.vpool != nullptr;
-    float* qs = lds;                       // [16][d]
-    float* ks = qs + LA_BQ * d;            // [KT][d + 1]
+    const int ldq = d + 1, ldps = KT + 1;  // odd strides: the four query rows of a wave read four different banks
+    float* qs = lds;                       // [16][d + 1]
+    float* ks = qs + LA_BQ * ldq;          // [KT][d + 1]
     float* vs = ks + KT * ldk;             // [KT][e], own value pages only
-    float* ps = vs + (ownv ? KT * e : 0);  // [16][KT]
+    float* ps = vs + (ownv ? KT * e : 0);  // [16][KT + 1]
     const float* vt = ownv ? vs : ks;
     const int ldv = ownv ? e : ldk;
     const int2 tile = a.tiles[blockIdx.x];
@@ -832,7 +833,7 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
     const int pos = sg.start_pos + lp;
     const int row = sg.row0 + lp;
     const int win = (int)min(a.win, 1ll << 30), keep = (int)min(a.keep, 1ll << 30), chunk = (int)min(a.chunk, 1ll << 30);
-    for (int i = ln; i < d; i += 16) qs[qr * d + i] = qvalid ? a.proj[(size_t)row * a.ldp + a.q_off + head * d + i] : 0.f;
+    for (int i = ln; i < d; i += 16) qs[qr * ldq + i] = qvalid ? a.proj[(size_t)row * a.ldp + a.q_off + head * d + i] : 0.f;
     const int pmin = sg.start_pos + q0 / nrep, pmax = sg.start_pos + (q0 + nq - 1) / nrep;
     int main_lo = max(0, pmin - win + 1);
     if (chunk > 0) main_lo = max(main_lo, pmin / chunk * chunk);
@@ -885,7 +886,7 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
             const int v = v0 + sl;
             const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
             float dot = 0.f;
-            for (int i = 0; i < d; ++i) dot = fmaf(qs[qr * d + i], ks[sl * ldk + i], dot);
+            for (int i = 0; i < d; ++i) dot = fmaf(qs[qr * ldq + i], ks[sl * ldk + i], dot);
             const int dist = pos - j;
             const bool vis = qvalid && v < total && dist >= 0 && ((dist < win && j >= clo) || j < keep);
             const float pen = a.bias == LBIAS_LOG ? r1 * log1pf(r2 * (float)dist) : r1 * (float)dist;
@@ -899,7 +900,7 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
 #pragma unroll
         for (int c = 0; c < KT / 16; ++c) {
             const float p = sc[c] == -INFINITY ? 0.f : expf(sc[c] - mn);
-            ps[qr * KT + ln + 16 * c] = p;
+            ps[qr * ldps + ln + 16 * c] = p;
             psum += p;
         }
         psum = row16_sum(psum);
@@ -912,7 +913,7 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
             const int i = ln + 16 * c;
             if (i < e) {
                 float o = acc[c] * corr;
-                for (int sl = 0; sl < kn; ++sl) o = fmaf(ps[qr * KT + sl], vt[sl * ldv + i], o);
+                for (int sl = 0; sl < kn; ++sl) o = fmaf(ps[qr * ldps + sl], vt[sl * ldv + i], o);
                 acc[c] = o;
             }
         }
@@ -1156,7 +1157,7 @@ __global__ __launch_bounds__(256) void lay_attn_merge_kernel(LAttnArgs a, int ns
     const int g = blockIdx.y, nrep = a.H / a.G, d = a.e;
     const int q0 = tile.y, nq = min(LA_BQ, sg.n * nrep - q0);
     const size_t t0 = ((size_t)blockIdx.x * a.G + g) * nsplit * LA_BQ;
-    for (int idx = threadIdx.x; idx < nq * d; idx += 256) {
+    for (int idx = blockIdx.z * 256 + threadIdx.x; idx < nq * d; idx += 256 * gridDim.z) {
         const int qr = idx / d, i = idx - qr * d;
         const int qi = q0 + qr, lp = qi / nrep, head = g * nrep + (qi - lp * nrep), row = sg.row0 + lp;
         float M = -INFINITY;
@@ -1176,8 +1177,9 @@ __global__ __launch_bounds__(256) void lay_attn_merge_kernel(LAttnArgs a, int ns
     }
 }
 static size_t lay_attn_lds(int d, int e, bool own_v, int KT) {
-    return (size_t)(LA_BQ * d + KT * (d + 1) + (own_v ? KT * e : 0) + LA_BQ * KT) * sizeof(float);
+    return (size_t)(LA_BQ * (d + 1) + KT * (d + 1) + (own_v ? KT * e : 0) + LA_BQ * (KT + 1)) * sizeof(float);
 }
+int lay_attn_key_tile(int d, int e, bool own_v);
 bool lay_attn_fits(int d, int e, bool own_v) {
     return d > 0 && e > 0 && e <= 512 && (own_v || e <= d) && lay_attn_lds(d, e, own_v, 32) <= LDS_MAX;
 }
@@ -1201,7 +1203,7 @@ void launch_lay_attn(const LAttnArgs& a0, int kvt, hipStream_t s) {
     const int nsplit = (a.part_o && a.part_ml && a.nsplit > 1) ? a.nsplit : 1;
     const dim3 grid((unsigned)a.ntiles, (unsigned)a.G, (unsigned)nsplit);
     // 64-key tiles where they stay inside 64 KiB of LDS (key head sizes up to 128 without value pages of their own), else 32
-    const bool narrow = a.d > 128 || lay_attn_lds(a.d, a.e, own_v, 64) > LDS_PLAIN;
+    const bool narrow = lay_attn_key_tile(a.d, a.e, own_v) == 32;
     const size_t lds = lay_attn_lds(a.d, a.e, own_v, narrow ? 32 : 64);
     const bool wide = a.e > 256;           // 32 output elements per lane instead of 16
     if (kvt == KV_F32) {
@@ -1213,8 +1215,12 @@ void launch_lay_attn(const LAttnArgs& a0, int kvt, hipStream_t s) {
         else if (narrow) lay_attn_go<KV_BF16, 32, 16>(a, grid, lds, s);
         else lay_attn_go<KV_BF16, 64, 16>(a, grid, lds, s);
     }
-    if (nsplit > 1) hipLaunchKernelGGL(lay_attn_merge_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G), dim3(256), 0, s, a, nsplit);
+    // the merge: one thread per output element, blocks of 256 over a tile's 16 rows
+    if (nsplit > 1)
+        hipLaunchKernelGGL(lay_attn_merge_kernel, dim3((unsigned)a.ntiles, (unsigned)a.G, (unsigned)std::max(1, std::min(16, LA_BQ * a.e / 1024))),
+                           dim3(256), 0, s, a, nsplit);
 }
+int lay_attn_key_tile(int d, int e, bool own_v) { return (d > 128 || lay_attn_lds(d, e, own_v, 64) > LDS_PLAIN) ? 32 : 64; }
 
 // ------------------------------------------------------------------------------------------------------------------
 // lightning attention: S_t = decay S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, per head, state [d][e] f32 per sequence.

@@ -167,6 +167,7 @@ void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int
                          const int32_t* rowseg, int T, int G, int d, int page, hipStream_t s);
 void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s);    // kvt: KV_BF16 | KV_F32
 bool lay_attn_fits(int d, int e, bool own_v);                         // sizes the kernel can hold in LDS and registers
+int lay_attn_key_tile(int d, int e, bool own_v);                      // keys per tile of lay_attn_kernel at these sizes (64 or 32)
 // bf16 key pages, d % 16 == 0, d <= 128: the matrix-core form; a.tiles lists {segment, first query row} in steps of
 // LAY_ATTN_MFMA_ROWS rows, longest key range first
 constexpr int LAY_ATTN_MFMA_ROWS = 64;

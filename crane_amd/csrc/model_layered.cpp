@@ -871,7 +871,8 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             {   // few query tiles and many visible keys (decode steps): share a tile's keys among blocks
                 long long seen = std::min<long long>(max_len, sp.win + sp.keep);
                 if (sp.chunk > 0) seen = std::min(seen, sp.chunk);
-                const int key_tiles = (int)((seen + 63) / 64), blocks = std::max(1, a.ntiles * sp.kv_heads);
+                const int kt = lay_attn_key_tile(dk, ev, a.vpool != nullptr);
+                const int key_tiles = (int)((seen + kt - 1) / kt), blocks = std::max(1, a.ntiles * sp.kv_heads);
                 a.nsplit = std::max(1, std::min({32, key_tiles, 256 / blocks, Layered::ATT_PARTS / blocks}));
                 a.part_o = L.att_po; a.part_ml = L.att_pml;
             }
