@@ -178,8 +178,8 @@ CONFIGS.update({
 # ---- layer-list decoders: Mononex ------------------------------------------------------------------------------------------
 def mononex_config(vocab: int, width: int, pattern: str, ff: int, heads: int, kv_heads: int, dim: int, vdim: int, block: int,
                    lat_heads: int, lat_dim: int, rot_dim: int, lat_vdim: int, kv_rank: int, q_rank: int,
-                   lin_heads: int, lin_dim: int, lin_vdim: int, tau: float = 16.0, rot_base: float = 500000.0,
-                   yarn: "dict | None" = None, eps: float = 1e-5) -> dict:
+                   lin_heads: int, lin_dim: int, lin_vdim: int, tau: float = 8.0, rot_base: float = 10000.0,
+                   yarn: "dict | None" = None, eps: float = 1e-6) -> dict:
     """pattern: one letter per layer -- 'a' softmax attention inside blocks of `block` positions, 'b' the same with the keys and
     values of the nearest 'a' before it, 'm' latent attention, 'g' gated linear attention; upper case: no feed-forward."""
     layers, last_a = [], None
