@@ -572,3 +572,54 @@ def test_gated_linear_attention_over_a_whole_pass_of_chunks(tmp_path):
         assert _err(got, want[rows]) < TOL_F32
     finally:
         m.close()
+
+
+def _drawn_config(seed):
+    """A model of this design with sizes, layer order and constants drawn from the seed (widths of a few hundred)."""
+    rs = np.random.RandomState(100 + seed)
+    pick = lambda *xs: xs[rs.randint(len(xs))]
+    width, layers, owners = pick(96, 128, 192, 256, 320), [], []
+    for i in range(rs.randint(4, 8)):
+        kind = pick("attention", "latent_attention", "gla")
+        mlp = None if rs.rand() < 0.2 else U.dense(pick(64, 136, 384, 512))
+        if kind == "attention":
+            if owners and rs.rand() < 0.5:
+                src = owners[rs.randint(len(owners))]
+                o = layers[src]["mixer"]
+                mx = U.attn(heads=o["kv_heads"] * pick(1, 2, 3), kv_heads=o["kv_heads"], dim=o["dim"], vdim=o["vdim"], size=pick(None, 17, 64, 100),
+                            scale=pick(0.1, 0.25), kv_from=src)
+            else:
+                kvh = pick(1, 2, 4)
+                mx = U.attn(heads=kvh * pick(1, 2, 4), kv_heads=kvh, dim=pick(16, 24, 32, 64), vdim=pick(16, 32, 48), size=pick(None, 30, 64, 128),
+                            scale=pick(0.125, 0.2))
+                owners.append(i)
+        elif kind == "latent_attention":
+            rot_dim = pick(8, 16, 32)
+            scaling = pick(None, dict(factor=pick(2.0, 8.0), original=pick(32, 128), fast=pick(8.0, 32.0), slow=pick(1.0, 2.0)))
+            mx = U.latent(heads=pick(1, 2, 4, 8), dim=pick(8, 16, 32), rot_dim=rot_dim, vdim=pick(16, 24, 32), kv_rank=pick(24, 64, 80, 128),
+                          q_rank=pick(32, 96, 128), scale=pick(0.1, 0.2), base=pick(100.0, 10000.0, 1e6), dims=pick(rot_dim, rot_dim // 2), scaling=scaling)
+        else:
+            mx = U.gla(heads=pick(1, 2, 4), dim=pick(8, 16, 32, 64), vdim=pick(16, 32, 64, 72), tau=pick(1.0, 4.0, 16.0, 32.0))
+        layers.append(U.layer(kind, mlp, **mx))
+    return U.config(layers, vocab=pick(97, 256, 601), width=width, eps=pick(1e-6, 1e-5, 1e-4))
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_models_whole_in_portions_and_decoded_in_both_formats(tmp_path, seed):
+    cfg = _drawn_config(seed)
+    P = U.random_weights(cfg, 30 + seed, a_rank=(4, 16, 24)[seed % 3])
+    toks = U.tokens(150, cfg["vocab"], 30 + seed)
+    want = O.forward(cfg, P, toks)
+    for dtype, tol in (("float32", TOL_F32), ("bfloat16", TOL_BF16)):
+        m = _load(tmp_path, cfg, P, dtype=dtype)
+        try:
+            a, b = m.seq_alloc(), m.seq_alloc()
+            whole, _ = m.step_batch([(a, toks, _all(150))])
+            assert _err(whole, want) < tol, (dtype, "whole")
+            out, at = [], 0
+            for c in [70, 2, 33, 1, 1, 17, 1, 25]:
+                out.append(m.step_batch([(b, toks[at:at + c], _all(c))])[0])
+                at += c
+            assert at == 150 and _err(np.concatenate(out), want) < tol, (dtype, "portions")
+        finally:
+            m.close()
